@@ -1,0 +1,16 @@
+"""MI355X-native KV-cache hot path of saragossa: thin Python host mirror over the C ABI.
+
+The product is ``libsaragossa_kv.so`` (hand-written gfx950 kernels behind
+``include/saragossa_kv.h``). This package only binds it with ctypes and mirrors
+the reference's Rust method names so the parity tests read like the reference's
+own tests. There is no CPU fallback: without the library, or without a GPU,
+every compute call raises.
+"""
+from ._lib import (KvError, DimensionError, ConfigError, DeviceError, lib, lib_path,
+                   DTYPE_BF16, DTYPE_F32, PAGE_ROWS)
+from .kv import DecodeResidentState, FullAttentionState
+from . import flags
+
+__all__ = ["KvError", "DimensionError", "ConfigError", "DeviceError", "lib", "lib_path",
+           "DecodeResidentState", "FullAttentionState", "flags", "DTYPE_BF16", "DTYPE_F32",
+           "PAGE_ROWS"]

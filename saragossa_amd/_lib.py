@@ -1,0 +1,115 @@
+"""ctypes loader for libsaragossa_kv.so. Fails loudly when the library is missing."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libsaragossa_kv.so")
+
+OK, ERR_DIMENSION, ERR_CONFIG, ERR_DEVICE = 0, 1, 2, 3
+DTYPE_F32, DTYPE_BF16 = 0, 1
+PAGE_ROWS = 16
+
+
+class KvError(RuntimeError):
+    """InferError of the reference (src/error.rs:12-75)."""
+
+    code = -1
+
+
+class DimensionError(KvError):
+    code = ERR_DIMENSION
+
+
+class ConfigError(KvError):
+    code = ERR_CONFIG
+
+
+class DeviceError(KvError):
+    code = ERR_DEVICE
+
+
+_BY_CODE = {ERR_DIMENSION: DimensionError, ERR_CONFIG: ConfigError, ERR_DEVICE: DeviceError}
+
+_lib = None
+
+_vp, _sz, _i32, _f32p = C.c_void_p, C.c_size_t, C.c_int32, C.POINTER(C.c_float)
+
+# name -> (restype, argtypes); every symbol include/saragossa_kv.h declares
+SIGNATURES = {
+    "skv_last_error": (C.c_char_p, []),
+    "skv_abi_version": (_i32, []),
+    "skv_env_flag": (_i32, [C.c_char_p, _i32]),
+    "skv_env_flag_value": (_i32, [C.c_char_p]),
+    "skv_flag_kv_bf16_for": (_i32, [_i32]),
+    "skv_flag_flash_sdpa_enabled": (_i32, []),
+    "skv_flag_sdpa_2pass_enabled": (_i32, []),
+    "skv_flag_sdpa_2pass_min_len": (_sz, []),
+    "skv_sdpa_2pass_blocks": (_sz, [_sz]),
+    "skv_flag_decode_resident_full": (_i32, []),
+    "skv_flag_decode_resident": (_i32, []),
+    "skv_flag_serve_prefix_cache_enabled": (_i32, []),
+    "skv_flag_serve_prefix_block_tokens": (_sz, []),
+    "skv_flag_serve_prefix_cache_blocks": (_sz, []),
+    "skv_flag_serve_prefix_blocks_per_session": (_sz, []),
+    "skv_flag_prefix_cache_enabled": (_i32, []),
+    "skv_flag_prefix_cache_capacity": (_sz, []),
+    "skv_flag_prefill_chunk": (_sz, []),
+    "skv_flags_reload": (None, []),
+    "skv_window_start": (_sz, [_sz, _sz]),
+    "skv_f32_to_bf16_bits": (C.c_uint16, [C.c_float]),
+    "skv_ctx_create": (_i32, [_i32, C.POINTER(_vp)]),
+    "skv_ctx_destroy": (None, [_vp]),
+    "skv_ctx_synchronize": (_i32, [_vp]),
+    "skv_layer_create": (_i32, [_vp, _sz, _sz, _sz, _sz, _i32, _sz, C.POINTER(_vp)]),
+    "skv_layer_create_for": (_i32, [_vp, _sz, _sz, _sz, _sz, _i32, C.POINTER(_vp)]),
+    "skv_layer_destroy": (None, [_vp]),
+    "skv_layer_set_block_table": (_i32, [_vp, _vp, _sz]),
+    "skv_layer_pages": (_sz, [_vp]),
+    "skv_kv_dim": (_sz, [_vp]),
+    "skv_len": (_sz, [_vp]),
+    "skv_capacity": (_sz, [_vp]),
+    "skv_q_heads": (_sz, [_vp]),
+    "skv_kv_heads": (_sz, [_vp]),
+    "skv_head_dim": (_sz, [_vp]),
+    "skv_window": (_sz, [_vp]),
+    "skv_logical_byte_len": (_sz, [_vp]),
+    "skv_truncate": (_i32, [_vp, _sz]),
+    "skv_seed": (_i32, [_vp, _vp, _vp, _sz, _sz]),
+    "skv_append_host": (_i32, [_vp, _vp, _vp, _sz]),
+    "skv_append_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz]),
+    "skv_append_batch_device": (_i32, [_vp, _vp, _vp, _vp, _sz]),
+    "skv_attention_host": (_i32, [_vp, _vp, _sz, _sz, _vp]),
+    "skv_attention_device": (_i32, [_vp, _vp, _vp, _vp, _sz]),
+    "skv_decode_step_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp]),
+    "skv_read_rows": (_i32, [_vp, _sz, _sz, _vp, _vp]),
+    "skv_gather_device": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp]),
+}
+
+
+def lib_path() -> str:
+    return _LIB
+
+
+def lib():
+    """The loaded library. Raises if it has not been built: there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            raise DeviceError(
+                f"{_LIB} is missing: build it with `python -c 'import __graft_entry__ as g; "
+                "g.build()'` (hipcc, gfx950). The KV path has no CPU fallback.")
+        l = C.CDLL(_LIB)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != OK:
+        msg = lib().skv_last_error().decode("utf-8", "replace")
+        raise _BY_CODE.get(rc, KvError)(msg)

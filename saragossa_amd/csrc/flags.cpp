@@ -1,0 +1,181 @@
+// Runtime kill-switches of the KV path, read from the environment like the
+// reference does (src/runtime_flags.rs:25-44; src/decode_resident/utils.rs:182-286).
+// Each getter is frozen at its first read; skv_flags_reload() drops the frozen
+// values and exists for tests only.
+#include <algorithm>
+#include <cctype>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <optional>
+#include <string>
+
+#include "skv_internal.h"
+
+namespace {
+
+std::mutex g_mu;
+uint64_t g_epoch = 1;
+
+std::string trim(const char *s) {
+    std::string v(s ? s : "");
+    size_t b = 0, e = v.size();
+    while (b < e && std::isspace((unsigned char)v[b])) ++b;
+    while (e > b && std::isspace((unsigned char)v[e - 1])) --e;
+    return v.substr(b, e - b);
+}
+
+bool ieq(const std::string &a, const char *b) {
+    if (a.size() != std::strlen(b)) return false;
+    for (size_t i = 0; i < a.size(); ++i)
+        if (std::tolower((unsigned char)a[i]) != b[i]) return false;
+    return true;
+}
+
+// env_flag_value (src/runtime_flags.rs:32-44)
+std::optional<bool> flag_value(const char *raw) {
+    const std::string v = trim(raw);
+    if (v == "1" || ieq(v, "true") || ieq(v, "on")) return true;
+    if (v == "0" || ieq(v, "false") || ieq(v, "off")) return false;
+    return std::nullopt;
+}
+
+bool env_flag(const char *name, bool dflt) {
+    const char *raw = std::getenv(name);
+    if (!raw) return dflt;
+    return flag_value(raw).value_or(dflt);
+}
+
+// value.trim().parse::<usize>().ok(): decimal digits only (an optional leading '+').
+std::optional<size_t> parse_usize(const char *raw, bool do_trim) {
+    if (!raw) return std::nullopt;
+    std::string v = do_trim ? trim(raw) : std::string(raw);
+    size_t i = 0;
+    if (!v.empty() && v[0] == '+') i = 1;
+    if (i >= v.size()) return std::nullopt;
+    size_t out = 0;
+    for (; i < v.size(); ++i) {
+        if (v[i] < '0' || v[i] > '9') return std::nullopt;
+        size_t d = (size_t)(v[i] - '0');
+        if (out > (SIZE_MAX - d) / 10) return std::nullopt;
+        out = out * 10 + d;
+    }
+    return out;
+}
+
+template <typename T> struct Once {
+    uint64_t epoch = 0;
+    T value{};
+    template <typename F> T get(F f) {
+        std::lock_guard<std::mutex> lk(g_mu);
+        if (epoch != g_epoch) {
+            value = f();
+            epoch = g_epoch;
+        }
+        return value;
+    }
+};
+
+Once<int> f_flash, f_2pass, f_res_full, f_res, f_serve_prefix, f_prefix, f_kv_bf16;
+Once<size_t> f_2pass_min, f_block_tokens, f_cache_blocks, f_per_session, f_prefix_cap, f_chunk;
+
+} // namespace
+
+extern "C" {
+
+int32_t skv_env_flag(const char *name, int32_t default_value) {
+    return env_flag(name, default_value != 0) ? 1 : 0;
+}
+
+int32_t skv_env_flag_value(const char *value) {
+    auto v = flag_value(value);
+    return v.has_value() ? (*v ? 1 : 0) : -1;
+}
+
+int32_t skv_flag_kv_bf16_for(int32_t sampled) {
+    // -1 = no override
+    int ov = f_kv_bf16.get([] {
+        const char *raw = std::getenv("RETI_RUST_KV_BF16");
+        if (!raw) return -1;
+        auto v = flag_value(raw);
+        return v.has_value() ? (*v ? 1 : 0) : -1;
+    });
+    return ov >= 0 ? ov : (sampled != 0);
+}
+
+int32_t skv_flag_flash_sdpa_enabled(void) {
+    return f_flash.get([] { return (int)env_flag("RETI_RUST_FLASH_SDPA", true); });
+}
+int32_t skv_flag_sdpa_2pass_enabled(void) {
+    return f_2pass.get([] { return (int)env_flag("RETI_RUST_SDPA_2PASS", true); });
+}
+size_t skv_flag_sdpa_2pass_min_len(void) {
+    // `.and_then(|value| value.parse().ok())`: no trim here in the reference.
+    return f_2pass_min.get([] {
+        return parse_usize(std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN"), false).value_or(2048);
+    });
+}
+size_t skv_sdpa_2pass_blocks(size_t len) {
+    size_t raw = std::max<size_t>(len / 128, 1);
+    size_t rounded = (raw + 31) / 32 * 32;
+    return std::min<size_t>(std::max<size_t>(rounded, 32), 1024);
+}
+int32_t skv_flag_decode_resident_full(void) {
+    return f_res_full.get([] { return (int)env_flag("RETI_RUST_DECODE_RESIDENT_FULL", true); });
+}
+int32_t skv_flag_decode_resident(void) {
+    return f_res.get([] { return (int)env_flag("RETI_RUST_DECODE_RESIDENT", false); });
+}
+int32_t skv_flag_serve_prefix_cache_enabled(void) {
+    return f_serve_prefix.get([] { return (int)env_flag("RETI_SERVE_PREFIX_CACHE", true); });
+}
+size_t skv_flag_serve_prefix_block_tokens(void) {
+    return f_block_tokens.get([] {
+        auto v = parse_usize(std::getenv("RETI_SERVE_PREFIX_BLOCK_TOKENS"), true);
+        return (v.has_value() && *v > 0) ? *v : (size_t)256;
+    });
+}
+size_t skv_flag_serve_prefix_cache_blocks(void) {
+    return f_cache_blocks.get(
+        [] { return parse_usize(std::getenv("RETI_SERVE_PREFIX_CACHE_BLOCKS"), true).value_or(128); });
+}
+size_t skv_flag_serve_prefix_blocks_per_session(void) {
+    size_t dflt = skv_flag_serve_prefix_cache_blocks();
+    return f_per_session.get([dflt] {
+        return parse_usize(std::getenv("RETI_SERVE_PREFIX_BLOCKS_PER_SESSION"), true).value_or(dflt);
+    });
+}
+int32_t skv_flag_prefix_cache_enabled(void) {
+    return f_prefix.get([] { return (int)env_flag("RETI_RUST_PREFIX_CACHE", true); });
+}
+size_t skv_flag_prefix_cache_capacity(void) {
+    return f_prefix_cap.get(
+        [] { return parse_usize(std::getenv("RETI_RUST_PREFIX_CACHE_CAP"), true).value_or(4); });
+}
+size_t skv_flag_prefill_chunk(void) {
+    return f_chunk.get([] {
+        // the alias is consulted only when the first variable is absent, not when it fails to parse
+        const char *raw = std::getenv("RETI_RUST_PREFILL_CHUNK");
+        if (!raw) raw = std::getenv("RETI_RUST_PREFILL_STEP_SIZE");
+        return parse_usize(raw, true).value_or(0);
+    });
+}
+
+void skv_flags_reload(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    ++g_epoch;
+}
+
+size_t skv_window_start(size_t position, size_t window) {
+    if (window == 0) return 0;
+    return position + 1 > window ? position + 1 - window : 0;
+}
+
+uint16_t skv_f32_to_bf16_bits(float value) {
+    uint32_t bits;
+    std::memcpy(&bits, &value, 4);
+    uint32_t lsb = (bits >> 16) & 1u;
+    return (uint16_t)((bits + 0x7fffu + lsb) >> 16);
+}
+
+} // extern "C"

@@ -1,0 +1,536 @@
+// Host side of one layer's paged KV cache: the stand-in for FullAttentionMetalState
+// (src/decode_resident/attention.rs:457-1038). All bookkeeping (len, block table)
+// lives on the host and advances at call time, before the GPU has run the work,
+// exactly like the reference's encode-time `len += 1` (attention.rs:993).
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "skv_internal.h"
+
+namespace skv {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+int32_t fail(int32_t code, const std::string &msg) {
+    g_last_error = msg;
+    return code;
+}
+int32_t fail_hip(hipError_t e, const char *what) {
+    g_last_error = std::string("HIP: ") + hipGetErrorString(e) + " (" + what + ")";
+    return SKV_ERR_DEVICE;
+}
+
+} // namespace skv
+
+using namespace skv;
+
+struct skv_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+};
+
+struct skv_layer {
+    skv_ctx *ctx = nullptr;
+    Geom g{};
+    size_t capacity = 0;
+    size_t len = 0;
+    size_t window = 0;    // 0 = full cache
+    size_t floor_pos = 0; // ring layers: oldest position still held
+    int n_pages = 0;
+    uint16_t *k_pool = nullptr;
+    uint16_t *v_pool = nullptr;
+    int32_t *table_dev = nullptr;
+    std::vector<int32_t> table;
+    // split-K partials
+    int max_splits = 1;
+    float *part_o = nullptr;
+    float *part_m = nullptr;
+    float *part_l = nullptr;
+    unsigned *counters = nullptr;
+    // staging for the synchronous host entry points
+    float *q_stage = nullptr;   // [q_dim]
+    float *out_stage = nullptr; // [q_dim]
+    float *kv_stage = nullptr;  // [2*kv_dim]
+    float *scores = nullptr;    // plain kernel: [q_heads][capacity], allocated on first use
+    size_t scores_cap = 0;
+};
+
+namespace {
+
+int padded_head_dim(size_t hd) {
+    for (int p : {32, 64, 128, 256, 512})
+        if ((size_t)p >= hd) return p;
+    return 0;
+}
+
+size_t env_usize(const char *name, size_t dflt) {
+    const char *raw = std::getenv(name);
+    if (!raw || !*raw) return dflt;
+    char *end = nullptr;
+    unsigned long long v = std::strtoull(raw, &end, 10);
+    if (end == raw) return dflt;
+    return (size_t)v;
+}
+
+// Rows below which the context is not split. The reference's default (2048,
+// src/decode_resident/utils.rs:270-278) was tuned for Apple GPUs; an explicit
+// RETI_RUST_SDPA_2PASS_MIN_LEN is honoured as is, the default here is 128 because a
+// single workgroup per kv head leaves 250 of the 256 compute units idle.
+size_t split_min_len() {
+    if (std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN")) return skv_flag_sdpa_2pass_min_len();
+    return 128;
+}
+
+int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows) {
+    if (!skv_flag_sdpa_2pass_enabled() || rows < split_min_len()) return 1;
+    const size_t target_wgs = env_usize("SKV_DECODE_WGS", 512);
+    const size_t min_pages = std::max<size_t>(env_usize("SKV_DECODE_MIN_PAGES", 4), 1);
+    size_t s = std::max<size_t>(target_wgs / (size_t)L->g.kv_heads, 1);
+    s = std::min<size_t>(s, (size_t)n_pages_scan / min_pages);
+    s = std::min<size_t>(s, (size_t)L->max_splits);
+    return (int)std::max<size_t>(s, 1);
+}
+
+hipStream_t as_stream(skv_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+int32_t check_window(const skv_layer *L, size_t window_start) {
+    if (L->len == 0) return fail(SKV_ERR_DIMENSION, "attention_decode sur KV vide");
+    if (window_start >= L->len)
+        return fail(SKV_ERR_DIMENSION, "attention_decode fenêtre vide: début=" +
+                                           std::to_string(window_start) +
+                                           ", len=" + std::to_string(L->len));
+    if (L->g.ring_rows > 0 && window_start < L->floor_pos)
+        return fail(SKV_ERR_DIMENSION,
+                    "attention_decode: fenêtre début=" + std::to_string(window_start) +
+                        " avant la plus ancienne ligne conservée " + std::to_string(L->floor_pos));
+    return SKV_OK;
+}
+
+int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float *out_dev,
+                         size_t window_start) {
+    int32_t rc = check_window(L, window_start);
+    if (rc) return rc;
+    const Geom &g = L->g;
+    const bool use_flash = skv_flag_flash_sdpa_enabled() && g.P <= 256;
+    if (!use_flash) {
+        const size_t need = (size_t)g.q_heads * L->capacity;
+        if (L->scores_cap < need) {
+            if (L->scores) {
+                SKV_HIP(hipDeviceSynchronize());
+                SKV_HIP(hipFree(L->scores));
+                L->scores = nullptr;
+                L->scores_cap = 0;
+            }
+            SKV_HIP(hipMalloc(&L->scores, need * sizeof(float)));
+            L->scores_cap = need;
+        }
+        NaiveArgs a{};
+        a.q = q_dev;
+        a.out = out_dev;
+        a.k_pool = L->k_pool;
+        a.v_pool = L->v_pool;
+        a.table = L->table_dev;
+        a.scores = L->scores;
+        a.len = (long)L->len;
+        a.window_start = (long)window_start;
+        a.inv_scale = 1.0f / std::sqrt((float)g.head_dim);
+        a.g = g;
+        SKV_HIP(launch_naive(a, s));
+        return SKV_OK;
+    }
+    DecodeArgs a{};
+    a.q = q_dev;
+    a.out = out_dev;
+    a.k_pool = L->k_pool;
+    a.v_pool = L->v_pool;
+    a.table = L->table_dev;
+    a.part_o = L->part_o;
+    a.part_m = L->part_m;
+    a.part_l = L->part_l;
+    a.counters = L->counters;
+    a.len = (long)L->len;
+    a.window_start = (long)window_start;
+    if (g.ring_rows > 0) {
+        a.page_first = 0;
+        a.n_pages = (int)std::min<size_t>((L->len + 15) / 16, (size_t)L->n_pages);
+    } else {
+        a.page_first = (int)(window_start / 16);
+        a.n_pages = (int)((L->len + 15) / 16) - a.page_first;
+    }
+    a.splits = choose_splits(L, a.n_pages, L->len - window_start);
+    // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
+    // 575); log2(e) moves the softmax to base 2.
+    a.qscale = (1.0f / std::sqrt((float)g.head_dim)) * 1.4426950408889634f;
+    a.g = g;
+    SKV_HIP(launch_decode(a, s));
+    return SKV_OK;
+}
+
+int32_t encode_append(skv_layer *L, hipStream_t s, const float *k_dev, const float *v_dev,
+                      size_t n_rows) {
+    if (n_rows == 0) return SKV_OK;
+    if (L->len + n_rows > L->capacity)
+        return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
+                                           std::to_string(L->capacity) + " atteinte (overflow)");
+    AppendArgs a{};
+    a.k_src = k_dev;
+    a.v_src = v_dev;
+    a.k_pool = L->k_pool;
+    a.v_pool = L->v_pool;
+    a.table = L->table_dev;
+    a.first_pos = (long)L->len;
+    a.n_rows = (int)n_rows;
+    a.g = L->g;
+    if (L->g.ring_rows > 0 && n_rows > (size_t)L->g.ring_rows) {
+        // only the last ring_rows rows survive; skip the ones that would be overwritten
+        const size_t skip = n_rows - (size_t)L->g.ring_rows;
+        const size_t kv_dim = (size_t)L->g.kv_heads * L->g.head_dim;
+        a.k_src += skip * kv_dim;
+        a.v_src += skip * kv_dim;
+        a.first_pos += (long)skip;
+        a.n_rows = L->g.ring_rows;
+    }
+    SKV_HIP(launch_append(a, s));
+    L->len += n_rows;
+    if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
+        L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
+    return SKV_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+const char *skv_last_error(void) { return g_last_error.c_str(); }
+int32_t skv_abi_version(void) { return 1; }
+
+int32_t skv_ctx_create(int32_t device, skv_ctx **out) {
+    if (!out) return fail(SKV_ERR_DEVICE, "skv_ctx_create: out nul");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(SKV_ERR_DEVICE, "aucun GPU HIP disponible (le chemin KV gfx950 exige un MI355X)");
+    if (device < 0 || device >= count)
+        return fail(SKV_ERR_CONFIG, "device " + std::to_string(device) + " hors plage");
+    SKV_HIP(hipSetDevice(device));
+    // The synchronous host entry points run on the legacy default stream, which
+    // orders itself against every blocking stream of the process (a framework's
+    // default stream included), so a host call that follows device-side calls on
+    // such a stream sees their effect without an explicit wait.
+    skv_ctx *c = new skv_ctx();
+    c->device = device;
+    c->stream = nullptr;
+    *out = c;
+    return SKV_OK;
+}
+
+void skv_ctx_destroy(skv_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    delete ctx;
+}
+
+int32_t skv_ctx_synchronize(skv_ctx *ctx) {
+    if (!ctx) return fail(SKV_ERR_DEVICE, "ctx nul");
+    SKV_HIP(hipStreamSynchronize(ctx->stream));
+    return SKV_OK;
+}
+
+void skv_layer_destroy(skv_layer *L) {
+    if (!L) return;
+    (void)hipSetDevice(L->ctx->device);
+    (void)hipDeviceSynchronize();
+    for (void *p : {(void *)L->k_pool, (void *)L->v_pool, (void *)L->table_dev, (void *)L->part_o,
+                    (void *)L->part_m, (void *)L->part_l, (void *)L->counters, (void *)L->q_stage,
+                    (void *)L->out_stage, (void *)L->kv_stage, (void *)L->scores})
+        if (p) (void)hipFree(p);
+    delete L;
+}
+
+int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
+                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) {
+    if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_layer_create: pointeur nul");
+    *out = nullptr;
+    if (capacity == 0 || q_heads == 0 || kv_heads == 0 || head_dim == 0)
+        return fail(SKV_ERR_CONFIG, "FullAttentionMetalState: dimension nulle");
+    if (q_heads % kv_heads != 0)
+        return fail(SKV_ERR_CONFIG, "GQA invalide: q_heads=" + std::to_string(q_heads) +
+                                        " non multiple de kv_heads=" + std::to_string(kv_heads));
+    if (dtype != SKV_DTYPE_BF16)
+        return fail(SKV_ERR_CONFIG, "KV f32 non construit dans cette bibliothèque: bf16 uniquement");
+    const int P = padded_head_dim(head_dim);
+    if (P == 0) return fail(SKV_ERR_CONFIG, "head_dim > 512 non supporté");
+    if (q_heads / kv_heads > 16)
+        return fail(SKV_ERR_CONFIG, "groupe GQA > 16 non supporté");
+    if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096)
+        return fail(SKV_ERR_CONFIG, "capacité KV déborde");
+    SKV_HIP(hipSetDevice(ctx->device));
+
+    skv_layer *L = new skv_layer();
+    L->ctx = ctx;
+    L->capacity = capacity;
+    L->window = window;
+    Geom &g = L->g;
+    g.q_heads = (int)q_heads;
+    g.kv_heads = (int)kv_heads;
+    g.head_dim = (int)head_dim;
+    g.P = P;
+    g.gqa = (int)(q_heads / kv_heads);
+    g.tile_elems = P * 16;
+    g.page_elems = (int)kv_heads * g.tile_elems;
+    size_t rows = capacity;
+    if (window > 0) {
+        const size_t ring = (window + 15) / 16 * 16;
+        g.ring_rows = (int)ring;
+        rows = ring;
+    }
+    L->n_pages = (int)((rows + 15) / 16);
+    const size_t pool_bytes = (size_t)L->n_pages * g.page_elems * sizeof(uint16_t);
+    const size_t q_dim = q_heads * head_dim;
+    const size_t kv_dim = kv_heads * head_dim;
+    L->max_splits = std::min(decode_max_splits(), std::max(1, L->n_pages));
+    const size_t n_part = (size_t)kv_heads * L->max_splits * g.gqa;
+
+    hipError_t e = hipSuccess;
+    auto alloc = [&](void **p, size_t bytes) {
+        if (e == hipSuccess) e = hipMalloc(p, bytes);
+    };
+    alloc((void **)&L->k_pool, pool_bytes);
+    alloc((void **)&L->v_pool, pool_bytes);
+    alloc((void **)&L->table_dev, (size_t)L->n_pages * sizeof(int32_t));
+    alloc((void **)&L->part_o, n_part * head_dim * sizeof(float));
+    alloc((void **)&L->part_m, n_part * sizeof(float));
+    alloc((void **)&L->part_l, n_part * sizeof(float));
+    alloc((void **)&L->counters, kv_heads * sizeof(unsigned));
+    alloc((void **)&L->q_stage, q_dim * sizeof(float));
+    alloc((void **)&L->out_stage, q_dim * sizeof(float));
+    alloc((void **)&L->kv_stage, 2 * kv_dim * sizeof(float));
+    // Padding dims and rows past `len` are multiplied by zero probabilities and zero
+    // query padding; they must hold finite values, so the pools start at zero.
+    if (e == hipSuccess) e = hipMemsetAsync(L->k_pool, 0, pool_bytes, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(L->v_pool, 0, pool_bytes, ctx->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(L->counters, 0, kv_heads * sizeof(unsigned), ctx->stream);
+    L->table.resize(L->n_pages);
+    for (int i = 0; i < L->n_pages; ++i) L->table[i] = i;
+    if (e == hipSuccess)
+        e = hipMemcpyAsync(L->table_dev, L->table.data(), (size_t)L->n_pages * sizeof(int32_t),
+                           hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        skv_layer_destroy(L);
+        return fail_hip(e, "allocation du cache KV");
+    }
+    *out = L;
+    return SKV_OK;
+}
+
+int32_t skv_layer_create_for(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
+                             size_t head_dim, int32_t sampled, skv_layer **out) {
+    const int32_t dtype = skv_flag_kv_bf16_for(sampled) ? SKV_DTYPE_BF16 : SKV_DTYPE_F32;
+    return skv_layer_create(ctx, capacity, q_heads, kv_heads, head_dim, dtype, 0, out);
+}
+
+int32_t skv_layer_set_block_table(skv_layer *L, const int32_t *table, size_t n) {
+    if (!L || !table) return fail(SKV_ERR_DEVICE, "set_block_table: pointeur nul");
+    if (L->len != 0) return fail(SKV_ERR_DIMENSION, "set_block_table: cache non vide");
+    if (n != (size_t)L->n_pages)
+        return fail(SKV_ERR_DIMENSION, "set_block_table: attendu " + std::to_string(L->n_pages) +
+                                           " entrées, reçu " + std::to_string(n));
+    std::vector<char> seen(n, 0);
+    for (size_t i = 0; i < n; ++i) {
+        if (table[i] < 0 || (size_t)table[i] >= n || seen[table[i]])
+            return fail(SKV_ERR_DIMENSION, "set_block_table: pas une permutation");
+        seen[table[i]] = 1;
+    }
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    L->table.assign(table, table + n);
+    SKV_HIP(hipMemcpyAsync(L->table_dev, L->table.data(), n * sizeof(int32_t), hipMemcpyHostToDevice,
+                           L->ctx->stream));
+    SKV_HIP(hipStreamSynchronize(L->ctx->stream));
+    return SKV_OK;
+}
+
+size_t skv_layer_pages(const skv_layer *L) { return L ? (size_t)L->n_pages : 0; }
+size_t skv_kv_dim(const skv_layer *L) { return L ? (size_t)L->g.kv_heads * L->g.head_dim : 0; }
+size_t skv_len(const skv_layer *L) { return L ? L->len : 0; }
+size_t skv_capacity(const skv_layer *L) { return L ? L->capacity : 0; }
+size_t skv_q_heads(const skv_layer *L) { return L ? (size_t)L->g.q_heads : 0; }
+size_t skv_kv_heads(const skv_layer *L) { return L ? (size_t)L->g.kv_heads : 0; }
+size_t skv_head_dim(const skv_layer *L) { return L ? (size_t)L->g.head_dim : 0; }
+size_t skv_window(const skv_layer *L) { return L ? L->window : 0; }
+size_t skv_logical_byte_len(const skv_layer *L) {
+    return L ? L->capacity * (size_t)L->g.kv_heads * L->g.head_dim * 2 : 0;
+}
+
+int32_t skv_truncate(skv_layer *L, size_t len) {
+    if (!L) return fail(SKV_ERR_DEVICE, "truncate: pointeur nul");
+    if (len > L->capacity)
+        return fail(SKV_ERR_DIMENSION, "truncate KV " + std::to_string(len) + " > capacité " +
+                                           std::to_string(L->capacity));
+    L->len = len;
+    if (len == 0) L->floor_pos = 0;
+    return SKV_OK;
+}
+
+int32_t skv_seed(skv_layer *L, const float *keys, const float *values, size_t n_elems,
+                 size_t n_rows) {
+    if (!L) return fail(SKV_ERR_DEVICE, "seed: pointeur nul");
+    if (n_rows > L->capacity)
+        return fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(n_rows) + " > capacité " +
+                                           std::to_string(L->capacity));
+    const size_t kv_dim = skv_kv_dim(L);
+    const size_t expected = n_rows * kv_dim;
+    if (n_elems != expected)
+        return fail(SKV_ERR_DIMENSION, "seed KV: attendu " + std::to_string(expected) + " (=" +
+                                           std::to_string(n_rows) + "×" + std::to_string(kv_dim) +
+                                           "), reçu " + std::to_string(n_elems));
+    if (n_rows > 0 && (!keys || !values)) return fail(SKV_ERR_DEVICE, "seed: pointeur nul");
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    L->len = 0;
+    L->floor_pos = 0;
+    if (n_rows == 0) return SKV_OK;
+    hipStream_t s = L->ctx->stream;
+    float *stage = nullptr;
+    SKV_HIP(hipMalloc((void **)&stage, 2 * expected * sizeof(float)));
+    hipError_t e = hipMemcpyAsync(stage, keys, expected * sizeof(float), hipMemcpyHostToDevice, s);
+    if (e == hipSuccess)
+        e = hipMemcpyAsync(stage + expected, values, expected * sizeof(float), hipMemcpyHostToDevice, s);
+    int32_t rc = SKV_OK;
+    if (e == hipSuccess) rc = encode_append(L, s, stage, stage + expected, n_rows);
+    hipError_t e2 = hipStreamSynchronize(s);
+    (void)hipFree(stage);
+    if (e != hipSuccess) return fail_hip(e, "seed: copie hôte→device");
+    if (rc) return rc;
+    if (e2 != hipSuccess) return fail_hip(e2, "seed: synchronisation");
+    return SKV_OK;
+}
+
+int32_t skv_append_host(skv_layer *L, const float *key, const float *value, size_t n_elems) {
+    if (!L || !key || !value) return fail(SKV_ERR_DEVICE, "append: pointeur nul");
+    const size_t kv_dim = skv_kv_dim(L);
+    if (n_elems != kv_dim)
+        return fail(SKV_ERR_DIMENSION, "append KV: attendu " + std::to_string(kv_dim) + ", reçu " +
+                                           std::to_string(n_elems));
+    if (L->len >= L->capacity)
+        return fail(SKV_ERR_DIMENSION,
+                    "append KV: capacité " + std::to_string(L->capacity) + " atteinte (overflow)");
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    hipStream_t s = L->ctx->stream;
+    SKV_HIP(hipMemcpyAsync(L->kv_stage, key, kv_dim * sizeof(float), hipMemcpyHostToDevice, s));
+    SKV_HIP(hipMemcpyAsync(L->kv_stage + kv_dim, value, kv_dim * sizeof(float), hipMemcpyHostToDevice, s));
+    int32_t rc = encode_append(L, s, L->kv_stage, L->kv_stage + kv_dim, 1);
+    if (rc) return rc;
+    SKV_HIP(hipStreamSynchronize(s));
+    return SKV_OK;
+}
+
+int32_t skv_append_device(skv_layer *L, skv_stream stream, const void *k_dev, size_t k_off,
+                          const void *v_dev, size_t v_off) {
+    if (!L || !k_dev || !v_dev) return fail(SKV_ERR_DEVICE, "append device: pointeur nul");
+    if ((k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "append device: offset non aligné f32");
+    return encode_append(L, as_stream(stream),
+                         reinterpret_cast<const float *>((const char *)k_dev + k_off),
+                         reinterpret_cast<const float *>((const char *)v_dev + v_off), 1);
+}
+
+int32_t skv_append_batch_device(skv_layer *L, skv_stream stream, const void *k_dev,
+                                const void *v_dev, size_t n_rows) {
+    if (!L || !k_dev || !v_dev) return fail(SKV_ERR_DEVICE, "append batch: pointeur nul");
+    if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "cache KV batch attend seq > 0");
+    return encode_append(L, as_stream(stream), (const float *)k_dev, (const float *)v_dev, n_rows);
+}
+
+int32_t skv_attention_device(skv_layer *L, skv_stream stream, const float *q_dev, float *out_dev,
+                             size_t window_start) {
+    if (!L || !q_dev || !out_dev) return fail(SKV_ERR_DEVICE, "attention device: pointeur nul");
+    return encode_attention(L, as_stream(stream), q_dev, out_dev, window_start);
+}
+
+int32_t skv_attention_host(skv_layer *L, const float *q, size_t n_elems, size_t window_start,
+                           float *out) {
+    if (!L || !q || !out) return fail(SKV_ERR_DEVICE, "attention: pointeur nul");
+    if (L->len == 0) return fail(SKV_ERR_DIMENSION, "attention_decode sur KV vide");
+    const size_t q_dim = (size_t)L->g.q_heads * L->g.head_dim;
+    if (n_elems != q_dim)
+        return fail(SKV_ERR_DIMENSION, "attention_decode: q attendu [" + std::to_string(q_dim) +
+                                           "], reçu " + std::to_string(n_elems));
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    hipStream_t s = L->ctx->stream;
+    SKV_HIP(hipMemcpyAsync(L->q_stage, q, q_dim * sizeof(float), hipMemcpyHostToDevice, s));
+    int32_t rc = encode_attention(L, s, L->q_stage, L->out_stage, window_start);
+    if (rc) return rc;
+    SKV_HIP(hipMemcpyAsync(out, L->out_stage, q_dim * sizeof(float), hipMemcpyDeviceToHost, s));
+    SKV_HIP(hipStreamSynchronize(s));
+    return SKV_OK;
+}
+
+int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_dev, size_t k_off,
+                               const void *v_dev, size_t v_off, const float *q_dev,
+                               float *out_dev) {
+    int32_t rc = skv_append_device(L, stream, k_dev, k_off, v_dev, v_off);
+    if (rc) return rc;
+    const size_t ws = skv_window_start(L->len - 1, L->window);
+    return skv_attention_device(L, stream, q_dev, out_dev, ws);
+}
+
+static int32_t check_rows(const skv_layer *L, size_t first, size_t n) {
+    if (first + n > L->len)
+        return fail(SKV_ERR_DIMENSION, "lecture KV lignes " + std::to_string(first) + ".." +
+                                           std::to_string(first + n) + " > len " +
+                                           std::to_string(L->len));
+    if (L->g.ring_rows > 0 && n > 0 && first < L->floor_pos)
+        return fail(SKV_ERR_DIMENSION, "lecture KV: ligne " + std::to_string(first) +
+                                           " déjà évincée de l'anneau");
+    return SKV_OK;
+}
+
+int32_t skv_gather_device(skv_layer *L, skv_stream stream, size_t first, size_t n, void *k_dst,
+                          void *v_dst) {
+    if (!L) return fail(SKV_ERR_DEVICE, "gather: pointeur nul");
+    int32_t rc = check_rows(L, first, n);
+    if (rc) return rc;
+    if (n == 0) return SKV_OK;
+    GatherArgs a{};
+    a.k_pool = L->k_pool;
+    a.v_pool = L->v_pool;
+    a.table = L->table_dev;
+    a.k_dst = (uint16_t *)k_dst;
+    a.v_dst = (uint16_t *)v_dst;
+    a.first_pos = (long)first;
+    a.n_rows = (int)n;
+    a.g = L->g;
+    SKV_HIP(launch_gather(a, as_stream(stream)));
+    return SKV_OK;
+}
+
+int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uint16_t *v_out) {
+    if (!L) return fail(SKV_ERR_DEVICE, "read_rows: pointeur nul");
+    int32_t rc = check_rows(L, first, n);
+    if (rc) return rc;
+    if (n == 0) return SKV_OK;
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    const size_t bytes = n * skv_kv_dim(L) * sizeof(uint16_t);
+    uint16_t *tmp = nullptr;
+    SKV_HIP(hipMalloc((void **)&tmp, 2 * bytes));
+    hipStream_t s = L->ctx->stream;
+    uint16_t *kd = tmp, *vd = tmp + n * skv_kv_dim(L);
+    rc = skv_gather_device(L, s, first, n, k_out ? kd : nullptr, v_out ? vd : nullptr);
+    hipError_t e = hipSuccess;
+    if (!rc && k_out) e = hipMemcpyAsync(k_out, kd, bytes, hipMemcpyDeviceToHost, s);
+    if (!rc && e == hipSuccess && v_out) e = hipMemcpyAsync(v_out, vd, bytes, hipMemcpyDeviceToHost, s);
+    hipError_t e2 = hipStreamSynchronize(s);
+    (void)hipFree(tmp);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail_hip(e, "read_rows: copie device→hôte");
+    if (e2 != hipSuccess) return fail_hip(e2, "read_rows: synchronisation");
+    return SKV_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,160 @@
+"""Host mirror of DecodeResidentState / FullAttentionMetalState over the C ABI.
+
+Method names follow src/decode_resident/attention.rs so that the parity tests
+read like src/decode_resident/tests.rs. Host entry points take numpy arrays;
+device entry points take raw device pointers (e.g. ``tensor.data_ptr()``) and a
+stream handle (e.g. ``torch.cuda.current_stream().cuda_stream``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from ._lib import DTYPE_BF16, check, lib
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class DecodeResidentState:
+    """DecodeResidentState::new (src/decoder/resident/setup.rs:237, 675)."""
+
+    def __init__(self, device: int = 0):
+        self._l = lib()
+        h = C.c_void_p()
+        check(self._l.skv_ctx_create(device, C.byref(h)))
+        self._h = h
+
+    def close(self) -> None:
+        if getattr(self, "_h", None):
+            self._l.skv_ctx_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def synchronize(self) -> None:
+        check(self._l.skv_ctx_synchronize(self._h))
+
+    def full_attention_with_element(self, capacity, q_heads, kv_heads, head_dim,
+                                    dtype=DTYPE_BF16, window=0) -> "FullAttentionState":
+        h = C.c_void_p()
+        check(self._l.skv_layer_create(self._h, capacity, q_heads, kv_heads, head_dim, dtype,
+                                       window, C.byref(h)))
+        return FullAttentionState(self, h)
+
+    def full_attention(self, capacity, q_heads, kv_heads, head_dim, sampled) -> "FullAttentionState":
+        """full_attention (src/decode_resident/attention.rs:26-45): dtype from the KV policy."""
+        h = C.c_void_p()
+        check(self._l.skv_layer_create_for(self._h, capacity, q_heads, kv_heads, head_dim,
+                                           int(sampled), C.byref(h)))
+        return FullAttentionState(self, h)
+
+    def full_attention_bf16(self, capacity, q_heads, kv_heads, head_dim, window=0):
+        """full_attention_bf16_for_test (attention.rs:47-54)."""
+        return self.full_attention_with_element(capacity, q_heads, kv_heads, head_dim,
+                                                DTYPE_BF16, window)
+
+
+class FullAttentionState:
+    """FullAttentionMetalState (src/decode_resident/attention.rs:457-1038). Not clonable."""
+
+    def __init__(self, ctx: DecodeResidentState, handle):
+        self._ctx = ctx  # keeps the context alive
+        self._l = ctx._l
+        self._h = handle
+
+    def close(self) -> None:
+        if getattr(self, "_h", None):
+            self._l.skv_layer_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def __copy__(self):
+        raise TypeError("device KV state is not clonable (src/decoder.rs:682-697)")
+
+    __deepcopy__ = __copy__
+
+    # ---- getters (attention.rs:485-548)
+    def kv_dim(self): return self._l.skv_kv_dim(self._h)
+    def len(self): return self._l.skv_len(self._h)
+    def __len__(self): return self.len()
+    def capacity(self): return self._l.skv_capacity(self._h)
+    def q_heads(self): return self._l.skv_q_heads(self._h)
+    def kv_heads(self): return self._l.skv_kv_heads(self._h)
+    def head_dim(self): return self._l.skv_head_dim(self._h)
+    def window(self): return self._l.skv_window(self._h)
+    def pages(self): return self._l.skv_layer_pages(self._h)
+    def byte_len(self): return self._l.skv_logical_byte_len(self._h)
+
+    def set_block_table(self, table) -> None:
+        t = np.ascontiguousarray(table, dtype=np.int32)
+        check(self._l.skv_layer_set_block_table(self._h, _p(t), t.size))
+
+    def truncate(self, n: int) -> None:
+        check(self._l.skv_truncate(self._h, n))
+
+    # ---- host entry points
+    def seed(self, keys_rows, values_rows, n_rows: int) -> None:
+        k, v = _f32(keys_rows).reshape(-1), _f32(values_rows).reshape(-1)
+        expected = n_rows * self.kv_dim()
+        n_elems = k.size if k.size != expected else v.size  # a wrong length reaches the check
+        check(self._l.skv_seed(self._h, _p(k), _p(v), n_elems, n_rows))
+
+    def append_row(self, key, value) -> None:
+        k, v = _f32(key).reshape(-1), _f32(value).reshape(-1)
+        n = k.size if k.size != self.kv_dim() else v.size  # a wrong length reaches the check
+        check(self._l.skv_append_host(self._h, _p(k), _p(v), n))
+
+    def attention_decode(self, q) -> np.ndarray:
+        return self.attention_decode_windowed(q, 0)
+
+    def attention_decode_windowed(self, q, window_start: int) -> np.ndarray:
+        qa = _f32(q).reshape(-1)
+        out = np.empty(self.q_heads() * self.head_dim(), dtype=np.float32)
+        check(self._l.skv_attention_host(self._h, _p(qa), qa.size, window_start, _p(out)))
+        return out
+
+    def read_rows(self, first: int = 0, n: int | None = None):
+        """Logical rows as bf16 bit patterns, ([n, kv_dim] uint16, same)."""
+        n = self.len() - first if n is None else n
+        k = np.empty((n, self.kv_dim()), dtype=np.uint16)
+        v = np.empty((n, self.kv_dim()), dtype=np.uint16)
+        check(self._l.skv_read_rows(self._h, first, n, _p(k), _p(v)))
+        return k, v
+
+    def read_rows_f32(self, first: int = 0, n: int | None = None):
+        k, v = self.read_rows(first, n)
+        return ((k.astype(np.uint32) << 16).view(np.float32),
+                (v.astype(np.uint32) << 16).view(np.float32))
+
+    # ---- device entry points (raw pointers + stream handle)
+    def encode_append_kv(self, stream, k_ptr, v_ptr) -> None:
+        self.encode_append_kv_with_offsets(stream, k_ptr, 0, v_ptr, 0)
+
+    def encode_append_kv_with_offsets(self, stream, k_ptr, k_off, v_ptr, v_off) -> None:
+        check(self._l.skv_append_device(self._h, stream, k_ptr, k_off, v_ptr, v_off))
+
+    def encode_append_batch(self, stream, k_ptr, v_ptr, n_rows) -> None:
+        check(self._l.skv_append_batch_device(self._h, stream, k_ptr, v_ptr, n_rows))
+
+    def encode_attention_decode(self, stream, q_ptr, out_ptr) -> None:
+        self.encode_attention_decode_windowed(stream, q_ptr, out_ptr, 0)
+
+    def encode_attention_decode_windowed(self, stream, q_ptr, out_ptr, window_start) -> None:
+        check(self._l.skv_attention_device(self._h, stream, q_ptr, out_ptr, window_start))
+
+    def encode_decode_step(self, stream, k_ptr, k_off, v_ptr, v_off, q_ptr, out_ptr) -> None:
+        check(self._l.skv_decode_step_device(self._h, stream, k_ptr, k_off, v_ptr, v_off, q_ptr,
+                                             out_ptr))
+
+    def encode_gather(self, stream, first, n, k_dst_ptr, v_dst_ptr) -> None:
+        check(self._l.skv_gather_device(self._h, stream, first, n, k_dst_ptr, v_dst_ptr))

@@ -1,0 +1,172 @@
+"""Cache-content parity on the GPU, restating the reference's KV tests
+(src/decode_resident/tests.rs:380-538, 1930-2018) against the paged bf16 cache.
+Contents are compared bit for bit with the oracle's bf16 rounding."""
+import numpy as np
+import pytest
+
+import oracle
+import saragossa_amd as skv
+from conftest import bf16_bits_to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+def test_kv_bf16_seed_then_append_rounds_to_bf16(state):
+    # src/decode_resident/tests.rs:435-478
+    q_heads, kv_heads, head_dim = 16, 2, 256
+    kv_dim = kv_heads * head_dim
+    capacity = 4
+    kv = state.full_attention_bf16(capacity, q_heads, kv_heads, head_dim)
+    assert kv.kv_dim() == kv_dim
+    assert kv.byte_len() == capacity * kv_dim * 2
+    seed_rows = 2
+    i = np.arange(seed_rows * kv_dim, dtype=np.float32)
+    seed_k = ((i - np.float32(333.0)) * np.float32(0.0017)).astype(np.float32)
+    seed_v = ((i + np.float32(17.0)) * np.float32(-0.0023)).astype(np.float32)
+    kv.seed(seed_k, seed_v, seed_rows)
+    c = np.arange(kv_dim, dtype=np.float32)
+    row_k = (np.float32(1.0) + c * np.float32(0.0009)).astype(np.float32)
+    row_v = (np.float32(-1.0) + c * np.float32(0.0011)).astype(np.float32)
+    kv.append_row(row_k, row_v)
+    assert kv.len() == seed_rows + 1
+    cpu_k = np.concatenate([seed_k, row_k])
+    cpu_v = np.concatenate([seed_v, row_v])
+    gk, gv = kv.read_rows()
+    assert np.array_equal(gk.reshape(-1), oracle.f32_to_bf16_bits(cpu_k))
+    assert np.array_equal(gv.reshape(-1), oracle.f32_to_bf16_bits(cpu_v))
+    assert np.array_equal(bf16_bits_to_f32(gk).reshape(-1), oracle.bf16_round(cpu_k))
+
+
+def test_kv_seed_then_append_matches_cpu(state):
+    # src/decode_resident/tests.rs:380-430, against the oracle cache in bf16-rounded mode
+    q_heads, kv_heads, head_dim = 16, 2, 256
+    kv_dim = kv_heads * head_dim
+    lay = oracle.layout(q_heads, kv_heads, head_dim)
+    kv = state.full_attention_bf16(6, q_heads, kv_heads, head_dim)
+    cpu = oracle.LayerKvCache("bf16r")
+    seed_rows = 3
+    idx = np.arange(seed_rows * kv_dim, dtype=np.float32)
+    seed_k = (idx * np.float32(0.001)).astype(np.float32)
+    seed_v = (idx * np.float32(-0.002) + np.float32(1.0)).astype(np.float32)
+    kv.seed(seed_k, seed_v, seed_rows)
+    cpu.append_batch(seed_k.reshape(seed_rows, kv_dim), seed_v.reshape(seed_rows, kv_dim), lay)
+    assert kv.len() == seed_rows
+    for r in range(seed_rows, seed_rows + 2):
+        c = (r * kv_dim + np.arange(kv_dim)).astype(np.float32)
+        k = (c * np.float32(0.003)).astype(np.float32)
+        v = (c * np.float32(0.004) - np.float32(0.5)).astype(np.float32)
+        kv.append_row(k, v)
+        cpu.append(k.reshape(1, -1), v.reshape(1, -1), lay)
+    assert kv.len() == seed_rows + 2 == len(cpu)
+    gk, gv = kv.read_rows_f32()
+    assert np.array_equal(gk, cpu.keys())
+    assert np.array_equal(gv, cpu.values())
+
+
+def test_kv_append_writes_at_nonzero_offset(state):
+    # src/decode_resident/tests.rs:482-503 (toy dims, kv_dim = 4)
+    kv = state.full_attention_bf16(4, 4, 2, 2)
+    kv.append_row([1.0, 2.0, 3.0, 4.0], [5.0, 6.0, 7.0, 8.0])
+    kv.append_row([10.0, 20.0, 30.0, 40.0], [50.0, 60.0, 70.0, 80.0])
+    gk, gv = kv.read_rows_f32()
+    assert gk.tolist() == [[1.0, 2.0, 3.0, 4.0], [10.0, 20.0, 30.0, 40.0]]
+    assert gv.tolist() == [[5.0, 6.0, 7.0, 8.0], [50.0, 60.0, 70.0, 80.0]]
+
+
+def test_kv_overflow_at_capacity_errors(state):
+    # src/decode_resident/tests.rs:507-525
+    q_heads, kv_heads, head_dim = 4, 2, 2
+    kv_dim = kv_heads * head_dim
+    prefill_len = 3
+    kv = state.full_attention_bf16(prefill_len, q_heads, kv_heads, head_dim)
+    seed = np.arange(prefill_len * kv_dim, dtype=np.float32)
+    kv.seed(seed, seed, prefill_len)
+    assert kv.len() == kv.capacity()
+    row = np.zeros(kv_dim, dtype=np.float32)
+    with pytest.raises(skv.DimensionError):
+        kv.append_row(row, row)
+    assert kv.len() == prefill_len
+
+
+def test_full_attention_state_rejects_non_multiple_gqa(state):
+    # src/decode_resident/tests.rs:528-538
+    with pytest.raises(skv.ConfigError):
+        state.full_attention_bf16(4, 3, 2, 8)
+
+
+def test_full_attention_state_rejects_zero_dims(state):
+    # src/decode_resident/attention.rs:64-68
+    for dims in [(0, 4, 2, 8), (4, 0, 2, 8), (4, 4, 0, 8), (4, 4, 2, 0)]:
+        with pytest.raises(skv.ConfigError):
+            state.full_attention_bf16(*dims)
+
+
+def test_seed_and_append_shape_errors(state):
+    # src/decode_resident/attention.rs:556-573, 613-619
+    kv = state.full_attention_bf16(4, 4, 2, 8)
+    kv_dim = 16
+    with pytest.raises(skv.DimensionError):
+        kv.seed(np.zeros(5 * kv_dim), np.zeros(5 * kv_dim), 5)  # n_rows > capacity
+    with pytest.raises(skv.DimensionError):
+        kv.seed(np.zeros(2 * kv_dim), np.zeros(2 * kv_dim - 1), 2)
+    with pytest.raises(skv.DimensionError):
+        kv.append_row(np.zeros(kv_dim - 1), np.zeros(kv_dim))
+    with pytest.raises(skv.DimensionError):
+        kv.truncate(5)
+    kv.truncate(0)
+
+
+@pytest.mark.parametrize("dims", [(32, 8, 128), (16, 2, 256), (4, 2, 16), (8, 8, 64), (6, 2, 96),
+                                  (2, 1, 40)])
+def test_paged_contents_with_permuted_block_table(state, dims):
+    """Logical row r lives at (block_table[r/16], r%16): seeding through a random permutation
+    and appending must read back bit-exact, and rows must land in the permuted pages."""
+    q_heads, kv_heads, head_dim = dims
+    kv_dim = kv_heads * head_dim
+    rng = np.random.default_rng(7)
+    capacity = 16 * 9 + 5
+    kv = state.full_attention_bf16(capacity, q_heads, kv_heads, head_dim)
+    table = rng.permutation(kv.pages()).astype(np.int32)
+    kv.set_block_table(table)
+    n = 16 * 7 + 3
+    k = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    v = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    kv.seed(k, v, n)
+    for _ in range(20):
+        kr = rng.standard_normal(kv_dim, dtype=np.float32)
+        vr = rng.standard_normal(kv_dim, dtype=np.float32)
+        kv.append_row(kr, vr)
+        k = np.vstack([k, kr[None]])
+        v = np.vstack([v, vr[None]])
+    gk, gv = kv.read_rows()
+    assert np.array_equal(gk, oracle.f32_to_bf16_bits(k))
+    assert np.array_equal(gv, oracle.f32_to_bf16_bits(v))
+    # partial reads through the table
+    gk2, gv2 = kv.read_rows(17, 40)
+    assert np.array_equal(gk2, gk[17:57]) and np.array_equal(gv2, gv[17:57])
+    # truncate drops rows without touching the kept ones
+    kv.truncate(33)
+    gk3, _ = kv.read_rows()
+    assert np.array_equal(gk3, gk[:33])
+    with pytest.raises(skv.DimensionError):
+        kv.read_rows(0, 34)
+
+
+def test_bf16_rounding_special_values(state):
+    """The device conversion is the reference's integer formula, including ties to even,
+    the carry into the exponent, infinities and the NaN non-special-case."""
+    vals = np.array([1.00390625, -0.33325195, 42.125, 0.0, -0.0, 1.0, 3.3895314e38, np.inf,
+                     -np.inf, 1.0039062, 1.0117188, 1e-40, -1e-45, 65504.0, 1.9960938,
+                     1.9980469, 0.1, -0.1], dtype=np.float32)
+    bits = np.array([0x7FC00000, 0x7F800001, 0xFFFFFFFF, 0x7FFF7FFF, 0x00008000, 0x00018000,
+                     0x00017FFF], dtype=np.uint32).view(np.float32)
+    vals = np.concatenate([vals, bits])
+    kv_dim = 32
+    pad = np.zeros(kv_dim - vals.size % kv_dim if vals.size % kv_dim else 0, dtype=np.float32)
+    data = np.concatenate([vals, pad]).reshape(-1, kv_dim)
+    kv = state.full_attention_bf16(data.shape[0], 1, 1, kv_dim)
+    kv.seed(data, data, data.shape[0])
+    gk, gv = kv.read_rows()
+    want = oracle.f32_to_bf16_bits(data)
+    assert np.array_equal(gk, want)
+    assert np.array_equal(gv, want)
