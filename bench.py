@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""KV-path decode benchmark on one MI355X.
+
+Workload (BASELINE.json configs[2]): a Qwen3.6-35B-A3B-style hybrid at 32k context.
+10 full-attention layers with 16 query heads, 2 KV heads, head_dim 256, bf16 KV in
+16-token pages behind random block tables, pre-filled with 32768 rows of N(0,1).
+One step = one decoded token: for each of the 10 layers, append one fresh K/V row
+and run paged GQA decode attention with a fresh query. Inputs are resident in HBM
+when the timed region starts.
+
+Prints ONE JSON line. `value` is microseconds per token over the 10 KV layers.
+`roofline` covers the decode attention kernel alone: algorithmic bytes per launch
+(K and V of one layer read once, query in, context out, block table) over the
+kernel's average duration measured with HIP events around every launch in a
+separate pass after the timed region. `cpu_baseline` times the CPU oracle (a C
+restatement of the reference's CPU path) on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+
+CFG = dict(layers=10, q_heads=16, kv_heads=2, head_dim=256, context=32768)
+
+
+def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> int:
+    """Bytes one layer's decode step has to move: K and V once (bf16), q in and ctx out
+    (f32), the block table, and the appended row when the append is counted."""
+    b = 2 * rows * kv_dim * 2 + 2 * q_dim * 4 + (rows + 15) // 16 * 4
+    if with_append:
+        b += 2 * kv_dim * 2
+    return b
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--context", type=int, default=CFG["context"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; every figure is one MI355X's throughput "
+              "(--gpus must be 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import saragossa_amd as skv
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the KV path has no CPU fallback", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    layers_n, qh, kvh, hd = CFG["layers"], CFG["q_heads"], CFG["kv_heads"], CFG["head_dim"]
+    kv_dim, q_dim = kvh * hd, qh * hd
+    ctx_rows = args.context
+    total_steps = args.warmup + args.steps
+    capacity = ctx_rows + 2 * total_steps + 8
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2)
+    rng = np.random.default_rng(2)
+    state = skv.DecodeResidentState(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    layers = []
+    host_kv = []  # first layer's f32 rows, kept for the CPU baseline
+    for li in range(layers_n):
+        kv = state.full_attention_bf16(capacity, qh, kvh, hd)
+        kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+        k = torch.randn(ctx_rows, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+        v = torch.randn(ctx_rows, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+        kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), ctx_rows)
+        torch.cuda.synchronize()
+        if li == 0 and not args.no_cpu_baseline:
+            host_kv = [k.cpu().numpy(), v.cpu().numpy()]
+        del k, v
+        layers.append(kv)
+
+    n_pass = 2 * total_steps  # timed pass + per-kernel pass
+    q_all = torch.randn(n_pass, layers_n, q_dim, device=dev, dtype=torch.float32, generator=gen)
+    k_all = torch.randn(n_pass, layers_n, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+    v_all = torch.randn(n_pass, layers_n, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+    out = torch.empty(layers_n, q_dim, device=dev, dtype=torch.float32)
+    torch.cuda.synchronize()
+
+    lib = skv.lib()
+    PtrArr = C.c_void_p * layers_n
+    layer_arr = PtrArr(*[l._h.value for l in layers])
+    out_arr = PtrArr(*[out[i].data_ptr() for i in range(layers_n)])
+
+    def ptrs(t, step):
+        base, stride = t[step].data_ptr(), t.stride(1) * 4
+        return PtrArr(*[base + i * stride for i in range(layers_n)])
+
+    step_ptrs = [(ptrs(k_all, s), ptrs(v_all, s), ptrs(q_all, s)) for s in range(n_pass)]
+
+    def run_step(s):
+        kp, vp, qp = step_ptrs[s]
+        rc = lib.skv_decode_step_layers_device(layer_arr, layers_n, stream, kp, vp, qp, out_arr)
+        if rc:
+            raise RuntimeError(lib.skv_last_error().decode())
+
+    for s in range(args.warmup):
+        run_step(s)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.warmup, total_steps):
+        run_step(s)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    us_per_token = ms_per_step * 1e3
+    rows_mid = ctx_rows + args.warmup + args.steps // 2
+    step_bytes = layers_n * algorithmic_bytes(rows_mid, kv_dim, q_dim, with_append=True)
+
+    # ---- per-kernel pass: HIP events around every attention launch, on the launch stream
+    evs = []
+    for s in range(total_steps, total_steps + args.steps):
+        kp, vp, qp = step_ptrs[s]
+        for li, kv in enumerate(layers):
+            kv.encode_append_kv(stream, kp[li], vp[li])
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            kv.encode_attention_decode(stream, qp[li], out_arr[li])
+            e1.record()
+            evs.append((e0, e1))
+    torch.cuda.synchronize()
+    kern_ms = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    kern_avg_us = sum(kern_ms) / len(kern_ms) * 1e3
+    kern_med_us = kern_ms[len(kern_ms) // 2] * 1e3
+    rows_k = ctx_rows + total_steps + args.steps // 2
+    launch_bytes = algorithmic_bytes(rows_k, kv_dim, q_dim, with_append=False)
+    achieved = launch_bytes / (kern_avg_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "KV-path decode us/token @32k ctx (append + paged GQA SDPA, 10 KV layers)",
+        "value": round(us_per_token, 2),
+        "unit": "us/token",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: 10 full-attention layers q16/kv2/hd256, bf16 KV in "
+                               "16-token pages, %d cached rows, batch 1, 1 token per step"
+                               % ctx_rows,
+                   "context": ctx_rows, "layers": layers_n, "page_rows": 16},
+        "tok_per_s": round(1e6 / us_per_token, 1),
+        "hbm_gbps": round(step_bytes / (us_per_token * 1e-6) / 1e9, 1),
+        "hbm_frac": round(step_bytes / (us_per_token * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel<256>",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": launch_bytes,
+                     "avg_launch_us": round(kern_avg_us, 2), "median_launch_us": round(kern_med_us, 2)},
+    }
+
+    if not args.no_cpu_baseline:
+        import oracle
+        threads = oracle.default_threads(qh)
+        lay = oracle.layout(qh, kvh, hd)
+        cache = oracle.LayerKvCache("f32")
+        cache.append_batch(host_kv[0], host_kv[1], lay)
+        kq = k_all[:, 0].cpu().numpy()
+        vq = v_all[:, 0].cpu().numpy()
+        qq = q_all[:, 0].cpu().numpy()
+        n_calls, t_cpu = 0, 0.0
+        budget = args.cpu_seconds
+        while t_cpu < budget and n_calls < kq.shape[0]:
+            c0 = time.perf_counter()
+            oracle.decode_step(cache, kq[n_calls], vq[n_calls], qq[n_calls], lay, threads)
+            t_cpu += time.perf_counter() - c0
+            n_calls += 1
+        cpu_us_per_token = t_cpu / n_calls * layers_n * 1e6
+        result["cpu_baseline"] = {
+            "value": round(cpu_us_per_token, 1), "unit": "us/token", "cores": threads,
+            "kind": "port",
+            "sample": "%d layer-steps of append + cached_attention_one on layer 0 (f32 cache, "
+                      "%d rows) timed and scaled by %d layers; host has %d cores"
+                      % (n_calls, ctx_rows, layers_n, os.cpu_count() or 0)}
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

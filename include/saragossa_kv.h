@@ -154,6 +154,16 @@ int32_t skv_decode_step_device(skv_layer *layer, skv_stream stream, const void *
                                size_t k_off, const void *v_dev, size_t v_off, const float *q_dev,
                                float *out_dev);
 
+/* The KV path of one token over several layers: for each layer i, append
+ * k_dev[i]/v_dev[i] (kv_dim f32 each) then attention of q_dev[i] into out_dev[i].
+ * It is the per-layer loop of enqueue_decode_token_resident
+ * (src/decoder/resident/decode.rs:183-458) restricted to the append and attention
+ * encodes, issued from native code so that a host in another language pays one
+ * FFI crossing per token instead of two per layer. */
+int32_t skv_decode_step_layers_device(skv_layer *const *layers, size_t n_layers, skv_stream stream,
+                                      const void *const *k_dev, const void *const *v_dev,
+                                      const float *const *q_dev, float *const *out_dev);
+
 /* Reads logical rows [first, first+n) through the block table as bf16 bits,
  * row-major [n, kv_dim]: the stand-in for reading keys()/values() back
  * (tests.rs:423-428, 469-476). Synchronous. */

@@ -1,0 +1,456 @@
+// gfx950 kernels of the KV hot path, part 2: split-K GQA decode attention over the
+// paged bf16 cache on the matrix cores, and the merge of its partials.
+#include "skv_internal.h"
+
+namespace skv {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+
+__device__ __forceinline__ uint16_t bf16_bits(float v) {
+    uint32_t b = __float_as_uint(v);
+    uint32_t lsb = (b >> 16) & 1u;
+    return (uint16_t)((b + 0x7fffu + lsb) >> 16);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+    return __uint_as_float(((uint32_t)b) << 16);
+}
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float xor_max(float v, int mask) {
+    return fmaxf(v, __shfl_xor(v, mask, 64));
+}
+
+constexpr int DEC_MAX_SPLITS = 512;
+int decode_max_splits() { return DEC_MAX_SPLITS; }
+
+// ------------------------------------------------------------------------------------
+// Decode attention, split-K over the context, one workgroup per (split, kv head).
+//
+// The GQA group's queries are staged once in LDS as bf16 hi + lo halves (q = hi + lo
+// to 2^-17), already multiplied by log2(e)/sqrt(head_dim). Each wavefront walks its
+// share of the pages. A 16-key K tile arrives as 1 KiB loads from consecutive addresses
+// and feeds S^T = K . Q^T on the matrix cores (16 keys x 16 query slots). The online
+// softmax, in base 2, runs on the accumulator registers: lane l holds keys
+// 4*(l/16)..+3 of query slot l%16, so the row maximum needs two cross-lane exchanges
+// and the row sum none until the end. The probabilities go straight back in as the B
+// operand of O^T += V^T . P^T, the V tile being stored transposed. Probabilities are
+// split hi + lo as well, so the result has fp32-level accuracy with bf16 operands.
+//
+// K registers are refilled right after the QK product that consumed them and V
+// registers right after the PV product, so each wavefront keeps about one page in
+// flight with a single K and a single V buffer; two wavefronts per SIMD hide the rest.
+//
+// At the end every wavefront writes its (o, m, l) to LDS and the whole workgroup
+// reduces them column-parallel: with one split that is the final context, otherwise a
+// partial per query head for the merge kernel.
+// ------------------------------------------------------------------------------------
+template <int KK>
+__device__ __forceinline__ void load_k(uint4 (&k)[KK], const DecodeArgs &a, int page, int kvh,
+                                       int lane) {
+    const long tile = (long)page * a.g.page_elems + (long)kvh * a.g.tile_elems;
+    const uint4 *kp = reinterpret_cast<const uint4 *>(a.k_pool + tile) + lane;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) k[kk] = kp[kk * 64];
+}
+template <int KK>
+__device__ __forceinline__ void load_v(uint4 (&v)[KK], const DecodeArgs &a, int page, int kvh,
+                                       int lane) {
+    const long tile = (long)page * a.g.page_elems + (long)kvh * a.g.tile_elems;
+    const uint4 *vp = reinterpret_cast<const uint4 *>(a.v_pool + tile) + lane;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) v[kk] = vp[kk * 64];
+}
+
+template <int P, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) {
+    constexpr int THREADS = WAVES * 64;
+    constexpr int KK = P / 32; // K-steps of the QK product, also column-tile pairs of V
+    constexpr int NT = P / 16; // 16-column tiles of the output
+    constexpr int OSTRIDE = P + 4;
+    const Geom g = a.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15; // key row inside the tile (A operand) / query slot (B, D)
+    const int j = lane >> 4;
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int G = g.gqa;
+
+    extern __shared__ __attribute__((aligned(16))) uint4 smem[];
+    uint4 *q_hi = smem;
+    uint4 *q_lo = smem + KK * 64;
+    uint16_t *new_k = reinterpret_cast<uint16_t *>(smem + 2 * KK * 64); // [P] appended row
+    uint16_t *new_v = new_k + P;
+
+    const int pb0 = a.page_first + (int)(((long)split * a.n_pages) / a.splits);
+    const int pb1 = a.page_first + (int)(((long)(split + 1) * a.n_pages) / a.splits);
+    // this wavefront walks pages pb0 + wave + it * WAVES, it = 0 .. n_it-1
+    const int n_it = pb1 - pb0 > wave ? (pb1 - pb0 - wave + WAVES - 1) / WAVES : 0;
+
+    // Fused append: the workgroup whose range holds the page of the new row rounds that
+    // row to bf16, stores it into the pools for later steps and keeps it in LDS; the
+    // wavefront that walks the page patches its registers from there, so nothing is read
+    // back from memory in this launch.
+    const int pb_new = a.new_slot >> 4;
+    const int r_new = a.new_slot & 15;
+    const bool appends = a.k_new != nullptr && pb_new >= pb0 && pb_new < pb1;
+    if (appends) {
+        const int page = a.table[pb_new];
+        const long tile = (long)page * g.page_elems + (long)kvh * g.tile_elems;
+        for (int d = tid; d < P; d += THREADS) {
+            uint16_t kb = 0, vb = 0;
+            if (d < g.head_dim) {
+                kb = bf16_bits(a.k_new[kvh * g.head_dim + d]);
+                vb = bf16_bits(a.v_new[kvh * g.head_dim + d]);
+                a.k_pool_w[tile + k_index(P, r_new, d)] = kb;
+                a.v_pool_w[tile + v_index(P, r_new, d)] = vb;
+            }
+            new_k[d] = kb;
+            new_v[d] = vb;
+        }
+    }
+
+    // Block-table entries of the next 64 iterations, one per lane.
+    int ids = 0;
+    auto fetch_ids = [&](int chunk) __attribute__((always_inline)) {
+        const int it = chunk * 64 + lane;
+        ids = it < n_it ? a.table[pb0 + wave + it * WAVES] : 0;
+    };
+    auto page_id = [&](int it) __attribute__((always_inline)) {
+        if ((it & 63) == 0 && it > 0) fetch_ids(it >> 6);
+        return __builtin_amdgcn_readlane(ids, it & 63);
+    };
+    fetch_ids(0);
+
+    // ---- queries of this kv head: load, start the first page, then stage to LDS ----------
+    constexpr int QI = (KK * 64 + THREADS - 1) / THREADS;
+    float qv[QI][8];
+#pragma unroll
+    for (int u = 0; u < QI; ++u) {
+        const int idx = min(tid + u * THREADS, KK * 64 - 1);
+        const int kk = idx >> 6;
+        const int jj = (idx >> 4) & 3;
+        const int qn = min(idx & 15, G - 1);
+        const float *qrow = a.q + (long)(kvh * G + qn) * g.head_dim;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[u][e] = qrow[min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
+    }
+    uint4 kr[KK], vr[KK];
+    if (n_it > 0) {
+        const int pg = page_id(0);
+        load_k<KK>(kr, a, pg, kvh, lane);
+        load_v<KK>(vr, a, pg, kvh, lane);
+    }
+#pragma unroll
+    for (int u = 0; u < QI; ++u) {
+        const int idx = tid + u * THREADS;
+        if (idx < KK * 64) {
+            const int kk = idx >> 6;
+            const int jj = (idx >> 4) & 3;
+            const bool row_ok = (idx & 15) < G;
+            uint32_t hi[4], lo[4];
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2) {
+                uint32_t h2 = 0, l2 = 0;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int d = kk * 32 + jj * 8 + e2 * 2 + h;
+                    const float v = (row_ok && d < g.head_dim) ? qv[u][e2 * 2 + h] * a.qscale : 0.0f;
+                    const uint16_t hb = bf16_bits(v);
+                    const uint16_t lb = bf16_bits(v - bf16_to_f32(hb));
+                    h2 |= (uint32_t)hb << (16 * h);
+                    l2 |= (uint32_t)lb << (16 * h);
+                }
+                hi[e2] = h2;
+                lo[e2] = l2;
+            }
+            q_hi[idx] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            q_lo[idx] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        }
+    }
+    __syncthreads();
+
+    float4_t o[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) o[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY; // running maximum of query slot n (same in the 4 lanes sharing n)
+    float l_run = 0.0f;      // this lane's share of the running sum
+
+    // S^T = K . Q^T for the page in kr: two independent accumulator chains (hi, lo halves)
+    auto qk = [&]() __attribute__((always_inline)) {
+        float4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const bf16x8_t kv = __builtin_bit_cast(bf16x8_t, kr[kk]);
+            const bf16x8_t qh = __builtin_bit_cast(bf16x8_t, q_hi[kk * 64 + lane]);
+            const bf16x8_t ql = __builtin_bit_cast(bf16x8_t, q_lo[kk * 64 + lane]);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, qh, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kv, ql, s1, 0, 0, 0);
+        }
+        return s0 + s1;
+    };
+    // online softmax step on the four scores of this lane; returns P^T as bf16 hi / lo
+    auto softmax_step = [&](float4_t s, int pb, short4_t &ph, short4_t &pl)
+                            __attribute__((always_inline)) {
+        // Only pages that touch the window start, the end of the cache or (ring layers) any
+        // page at all can hold keys outside [window_start, len).
+        const int first_slot = pb * 16;
+        const bool interior = g.ring_rows == 0 && first_slot >= a.window_start &&
+                              first_slot + 16 <= a.len;
+        if (!interior) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int slot = first_slot + j * 4 + i;
+                int pos = slot;
+                if (g.ring_rows > 0)
+                    pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+                const bool ok = pos >= a.window_start && pos < a.len;
+                s[i] = ok ? s[i] : -INFINITY;
+            }
+        }
+        float m_blk = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+        m_blk = xor_max(m_blk, 16);
+        m_blk = xor_max(m_blk, 32);
+        const float m_new = fmaxf(m_run, m_blk);
+        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        float psum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float p = fast_exp2(s[i] - m_safe);
+            psum += p;
+            const uint16_t hb = bf16_bits(p);
+            const uint16_t lb = bf16_bits(p - bf16_to_f32(hb));
+            ph[i] = (short)hb;
+            pl[i] = (short)lb;
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) o[t] *= alpha;
+        }
+    };
+    auto pv = [&](short4_t ph, short4_t pl) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const short4_t v0 = __builtin_bit_cast(short4_t, make_uint2(vr[kk].x, vr[kk].y));
+            const short4_t v1 = __builtin_bit_cast(short4_t, make_uint2(vr[kk].z, vr[kk].w));
+            o[2 * kk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v0, ph, o[2 * kk], 0, 0, 0);
+            o[2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v1, ph, o[2 * kk + 1], 0, 0, 0);
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const short4_t v0 = __builtin_bit_cast(short4_t, make_uint2(vr[kk].x, vr[kk].y));
+            const short4_t v1 = __builtin_bit_cast(short4_t, make_uint2(vr[kk].z, vr[kk].w));
+            o[2 * kk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v0, pl, o[2 * kk], 0, 0, 0);
+            o[2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v1, pl, o[2 * kk + 1], 0, 0, 0);
+        }
+    };
+
+    // the page that receives the appended row takes it from LDS instead of memory
+    auto patch_k = [&](int pb) __attribute__((always_inline)) {
+        if (appends && pb == pb_new && n == r_new) {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk)
+                kr[kk] = *reinterpret_cast<const uint4 *>(new_k + kk * 32 + j * 8);
+        }
+    };
+    auto patch_v = [&](int pb) __attribute__((always_inline)) {
+        if (appends && pb == pb_new && j == (r_new >> 2)) {
+            const int i = r_new & 3;
+            const uint32_t keep = (i & 1) ? 0x0000ffffu : 0xffff0000u;
+            const int sh = (i & 1) * 16;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                const uint32_t b0 = (uint32_t)new_v[kk * 32 + n] << sh;
+                const uint32_t b1 = (uint32_t)new_v[kk * 32 + 16 + n] << sh;
+                if (i < 2) {
+                    vr[kk].x = (vr[kk].x & keep) | b0;
+                    vr[kk].z = (vr[kk].z & keep) | b1;
+                } else {
+                    vr[kk].y = (vr[kk].y & keep) | b0;
+                    vr[kk].w = (vr[kk].w & keep) | b1;
+                }
+            }
+        }
+    };
+
+    // Steady state is unconditional (the compiler can then wait for exactly the loads it
+    // needs); the last page is peeled.
+    for (int it = 0; it + 1 < n_it; ++it) {
+        const int pb = pb0 + wave + it * WAVES;
+        const int next = page_id(it + 1);
+        patch_k(pb);
+        const float4_t s = qk();
+        load_k<KK>(kr, a, next, kvh, lane);
+        short4_t ph, pl;
+        softmax_step(s, pb, ph, pl);
+        patch_v(pb);
+        pv(ph, pl);
+        load_v<KK>(vr, a, next, kvh, lane);
+    }
+    if (n_it > 0) {
+        const int pb = pb0 + wave + (n_it - 1) * WAVES;
+        patch_k(pb);
+        const float4_t s = qk();
+        short4_t ph, pl;
+        softmax_step(s, pb, ph, pl);
+        patch_v(pb);
+        pv(ph, pl);
+    }
+
+    // this lane's share of the sum -> the query slot's sum
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+
+    // ---- all wavefronts publish (o, m, l); the workgroup reduces them column-parallel -------
+    __syncthreads(); // the staged queries are no longer needed: the LDS is reused
+    float *xo = reinterpret_cast<float *>(smem);        // [WAVES][G][OSTRIDE]
+    float *xm = xo + WAVES * G * OSTRIDE;               // [WAVES][G]
+    float *xl = xm + WAVES * G;                         // [WAVES][G]
+    if (n < G) {
+        float *dst = xo + (wave * G + n) * OSTRIDE + j * 4;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) *reinterpret_cast<float4_t *>(dst + t * 16) = o[t];
+        if (j == 0) {
+            xm[wave * G + n] = m_run;
+            xl[wave * G + n] = l_run;
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < G * P; idx += THREADS) {
+        const int row = idx / P;
+        const int col = idx - row * P;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, xm[w * G + row]);
+        const float m_safe = mx == -INFINITY ? 0.0f : mx;
+        float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float wgt = fast_exp2(xm[w * G + row] - m_safe);
+            acc += wgt * xo[(w * G + row) * OSTRIDE + col];
+            lsum += wgt * xl[w * G + row];
+        }
+        if (col < g.head_dim) {
+            if (a.splits == 1) {
+                a.out[(long)(kvh * G + row) * g.head_dim + col] = acc / lsum;
+            } else {
+                const long pidx = ((long)kvh * a.splits + split) * G + row;
+                a.part_o[pidx * g.head_dim + col] = acc;
+                if (col == 0) {
+                    a.part_m[pidx] = mx;
+                    a.part_l[pidx] = lsum;
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// Merge of the split-K partials: one workgroup per (query head, 16 columns). The 256
+// threads are 16 columns x 16 split lanes. Every thread issues all its loads (o, m, l
+// of its splits) at once, so the kernel costs one round trip to memory; the maximum
+// and the two sums are then reduced across the split lanes through LDS.
+// Stands in for attention_decode_2pass_2 (src/decode_resident/kernels.rs:801-917).
+// ------------------------------------------------------------------------------------
+constexpr int MERGE_PER_LANE = DEC_MAX_SPLITS / 16;
+
+__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
+    const Geom g = a.g;
+    const int h = blockIdx.x;
+    const int kvh = h / g.gqa;
+    const int gq = h - kvh * g.gqa;
+    const int tid = threadIdx.x;
+    const int c = tid & 15;
+    const int col = min(blockIdx.y * 16 + c, g.head_dim - 1);
+    const int sl = tid >> 4;
+    __shared__ float red_m[16];
+    __shared__ float red_l[16];
+    __shared__ float acc_x[16][17];
+    const long base = ((long)kvh * a.splits) * g.gqa + gq;
+    const long ostride = (long)g.gqa * g.head_dim;
+    const float *po = a.part_o + base * g.head_dim + col;
+    float ov[MERGE_PER_LANE], mv[MERGE_PER_LANE], lv[MERGE_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < MERGE_PER_LANE; ++i) {
+        const int s = sl + 16 * i;
+        const bool ok = s < a.splits;
+        const int sc = ok ? s : 0;
+        mv[i] = a.part_m[base + (long)sc * g.gqa];
+        lv[i] = a.part_l[base + (long)sc * g.gqa];
+        ov[i] = po[(long)sc * ostride];
+        if (!ok) {
+            mv[i] = -INFINITY;
+            lv[i] = 0.0f;
+            ov[i] = 0.0f;
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < MERGE_PER_LANE; ++i) mx = fmaxf(mx, mv[i]);
+    if (c == 0) red_m[sl] = mx;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, red_m[i]);
+    const float m_safe = mx == -INFINITY ? 0.0f : mx;
+    float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MERGE_PER_LANE; ++i) {
+        const float w = fast_exp2(mv[i] - m_safe);
+        acc += w * ov[i];
+        lsum += w * lv[i];
+    }
+    acc_x[sl][c] = acc;
+    if (c == 0) red_l[sl] = lsum;
+    __syncthreads();
+    if (sl == 0 && (int)blockIdx.y * 16 + c < g.head_dim) {
+        float t = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            t += acc_x[i][c];
+            l += red_l[i];
+        }
+        a.out[(long)h * g.head_dim + col] = t / l;
+    }
+}
+
+template <int P, int WAVES>
+static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
+    constexpr int KK = P / 32;
+    const size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
+    const size_t xchg = ((size_t)WAVES * a.g.gqa * (P + 4) + 2 * WAVES * a.g.gqa) * sizeof(float);
+    const size_t lds = stage > xchg ? stage : xchg;
+    static bool attr_set = false; // per instantiation
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads);
+    hipLaunchKernelGGL((decode_split_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
+    hipError_t e = hipErrorInvalidValue;
+    const bool w8 = a.waves == 8;
+    switch (a.g.P) {
+    case 32: e = w8 ? launch_split<32, 8>(a, s) : launch_split<32, 4>(a, s); break;
+    case 64: e = w8 ? launch_split<64, 8>(a, s) : launch_split<64, 4>(a, s); break;
+    case 128: e = w8 ? launch_split<128, 8>(a, s) : launch_split<128, 4>(a, s); break;
+    case 256: e = w8 ? launch_split<256, 8>(a, s) : launch_split<256, 4>(a, s); break;
+    default: break;
+    }
+    if (e != hipSuccess || a.splits == 1) return e;
+    dim3 mgrid((unsigned)a.g.q_heads, (unsigned)((a.g.head_dim + 15) / 16));
+    hipLaunchKernelGGL(decode_merge_kernel, mgrid, dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+} // namespace skv

@@ -86,10 +86,18 @@ size_t split_min_len() {
     return 128;
 }
 
-int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows) {
+// Wavefronts per workgroup of the split kernel. Eight halve the number of partials
+// for the same number of wavefronts in flight.
+int choose_waves(const skv_layer *L) {
+    const size_t w = env_usize("SKV_DECODE_WAVES", 8);
+    (void)L;
+    return w == 4 ? 4 : 8;
+}
+
+int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows, int waves) {
     if (!skv_flag_sdpa_2pass_enabled() || rows < split_min_len()) return 1;
-    const size_t target_wgs = env_usize("SKV_DECODE_WGS", 512);
-    const size_t min_pages = std::max<size_t>(env_usize("SKV_DECODE_MIN_PAGES", 4), 1);
+    const size_t target_wgs = env_usize("SKV_DECODE_WGS", 256);
+    const size_t min_pages = std::max<size_t>(env_usize("SKV_DECODE_MIN_PAGES", (size_t)waves), 1);
     size_t s = std::max<size_t>(target_wgs / (size_t)L->g.kv_heads, 1);
     s = std::min<size_t>(s, (size_t)n_pages_scan / min_pages);
     s = std::min<size_t>(s, (size_t)L->max_splits);
@@ -111,12 +119,17 @@ int32_t check_window(const skv_layer *L, size_t window_start) {
     return SKV_OK;
 }
 
+bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L->g.P <= 256; }
+
+// k_new / v_new non-null: the row at position len-1 has not been written yet and the
+// attention kernel appends it itself (the host bookkeeping has already advanced).
 int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float *out_dev,
-                         size_t window_start) {
+                         size_t window_start, const float *k_new = nullptr,
+                         const float *v_new = nullptr) {
     int32_t rc = check_window(L, window_start);
     if (rc) return rc;
     const Geom &g = L->g;
-    const bool use_flash = skv_flag_flash_sdpa_enabled() && g.P <= 256;
+    const bool use_flash = uses_flash(L);
     if (!use_flash) {
         const size_t need = (size_t)g.q_heads * L->capacity;
         if (L->scores_cap < need) {
@@ -152,20 +165,27 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     a.part_o = L->part_o;
     a.part_m = L->part_m;
     a.part_l = L->part_l;
-    a.counters = L->counters;
-    a.len = (long)L->len;
-    a.window_start = (long)window_start;
+    a.len = (int)L->len;
+    a.window_start = (int)window_start;
     if (g.ring_rows > 0) {
         a.page_first = 0;
         a.n_pages = (int)std::min<size_t>((L->len + 15) / 16, (size_t)L->n_pages);
+        a.ring_t = (int)((L->len - 1) % (size_t)g.ring_rows);
+        a.ring_base = (int)(L->len - 1) - a.ring_t;
     } else {
         a.page_first = (int)(window_start / 16);
         a.n_pages = (int)((L->len + 15) / 16) - a.page_first;
     }
-    a.splits = choose_splits(L, a.n_pages, L->len - window_start);
+    a.waves = choose_waves(L);
+    a.splits = choose_splits(L, a.n_pages, L->len - window_start, a.waves);
     // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
     // 575); log2(e) moves the softmax to base 2.
     a.qscale = (1.0f / std::sqrt((float)g.head_dim)) * 1.4426950408889634f;
+    a.k_new = k_new;
+    a.v_new = v_new;
+    a.k_pool_w = L->k_pool;
+    a.v_pool_w = L->v_pool;
+    a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
     a.g = g;
     SKV_HIP(launch_decode(a, s));
     return SKV_OK;
@@ -474,10 +494,42 @@ int32_t skv_attention_host(skv_layer *L, const float *q, size_t n_elems, size_t 
 int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_dev, size_t k_off,
                                const void *v_dev, size_t v_off, const float *q_dev,
                                float *out_dev) {
-    int32_t rc = skv_append_device(L, stream, k_dev, k_off, v_dev, v_off);
-    if (rc) return rc;
+    if (!L || !k_dev || !v_dev || !q_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step: pointeur nul");
+    static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
+    if (!fused || !uses_flash(L)) {
+        int32_t rc = skv_append_device(L, stream, k_dev, k_off, v_dev, v_off);
+        if (rc) return rc;
+        const size_t ws = skv_window_start(L->len - 1, L->window);
+        return skv_attention_device(L, stream, q_dev, out_dev, ws);
+    }
+    if ((k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "append device: offset non aligné f32");
+    if (L->len >= L->capacity)
+        return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
+                                           std::to_string(L->capacity) + " atteinte (overflow)");
+    // the attention kernel writes the row itself: advance the bookkeeping first
+    L->len += 1;
+    if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
+        L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
     const size_t ws = skv_window_start(L->len - 1, L->window);
-    return skv_attention_device(L, stream, q_dev, out_dev, ws);
+    int32_t rc = encode_attention(L, as_stream(stream), q_dev, out_dev, ws,
+                                  reinterpret_cast<const float *>((const char *)k_dev + k_off),
+                                  reinterpret_cast<const float *>((const char *)v_dev + v_off));
+    if (rc) L->len -= 1;
+    return rc;
+}
+
+int32_t skv_decode_step_layers_device(skv_layer *const *layers, size_t n_layers, skv_stream stream,
+                                      const void *const *k_dev, const void *const *v_dev,
+                                      const float *const *q_dev, float *const *out_dev) {
+    if (!layers || !k_dev || !v_dev || !q_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step_layers: pointeur nul");
+    for (size_t i = 0; i < n_layers; ++i) {
+        int32_t rc = skv_decode_step_device(layers[i], stream, k_dev[i], 0, v_dev[i], 0, q_dev[i],
+                                            out_dev[i]);
+        if (rc) return rc;
+    }
+    return SKV_OK;
 }
 
 static int32_t check_rows(const skv_layer *L, size_t first, size_t n) {

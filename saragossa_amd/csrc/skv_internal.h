@@ -92,18 +92,21 @@ struct DecodeArgs {
     float *part_o;   // [kv_heads][splits][gqa][head_dim]
     float *part_m;   // [kv_heads][splits][gqa]   (log2 domain)
     float *part_l;   // [kv_heads][splits][gqa]
-    unsigned *counters; // [kv_heads] arrival counters for the fused merge (zero between launches)
-    long len;          // rows valid (positions 0..len)
-    long window_start; // first position attended
-    int page_first;    // first logical page scanned
-    int n_pages;       // logical pages scanned
+    int len;          // rows valid: positions 0..len
+    int window_start; // first position attended
+    int ring_base;    // ring layers: (len-1) - (len-1) % ring_rows
+    int ring_t;       // ring layers: (len-1) % ring_rows
+    int page_first;   // first logical page scanned
+    int n_pages;      // logical pages scanned
     int splits;
-    float qscale;      // (1/sqrt(head_dim)) * log2(e)
-    // optional fused append of the row at position len-1 (null = none)
-    const float *k_new;
+    int waves;        // wavefronts per workgroup: 4 or 8
+    float qscale;     // (1/sqrt(head_dim)) * log2(e)
+    // fused append of the row at position len-1 (k_new null = none)
+    const float *k_new; // [kv_dim] f32
     const float *v_new;
     uint16_t *k_pool_w;
     uint16_t *v_pool_w;
+    int new_slot;     // slot that receives the row
     Geom g;
 };
 
