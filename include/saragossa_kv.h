@@ -172,6 +172,119 @@ int32_t skv_read_rows(skv_layer *layer, size_t first, size_t n, uint16_t *k_out,
 int32_t skv_gather_device(skv_layer *layer, skv_stream stream, size_t first, size_t n,
                           void *k_dst_dev, void *v_dst_dev);
 
+/* ---- block snapshots: snapshot/copy/restore_prompt_state_metal ------------- */
+
+/* Deep copy of logical blocks (16-row pages) `block_ids` of every layer into storage the
+ * snapshot owns: the block-paged form of snapshot_prompt_state_metal
+ * (src/decoder/generation.rs:2834-2849). Async on `stream`. */
+int32_t skv_snapshot_blocks(skv_ctx *ctx, skv_stream stream, skv_layer *const *layers,
+                            size_t n_layers, const size_t *block_ids, size_t n_blocks,
+                            skv_snapshot **out);
+/* copy_prompt_state_metal_snapshot (generation.rs:2856-2871): an independent copy, so that
+ * restoring never aliases the cached entry (src/serve/state.rs:580-584). */
+int32_t skv_snapshot_clone(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snapshot,
+                           skv_snapshot **out);
+/* restore_prompt_state_metal (generation.rs:2878-2892): block i of the snapshot goes to
+ * logical block dst_block_ids[i] of every layer; SKV_ERR_DIMENSION when the layer count
+ * or shapes differ (generation.rs:3086-3092). The caller sets the length with skv_truncate. */
+int32_t skv_restore_blocks(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snapshot,
+                           skv_layer *const *layers, size_t n_layers, const size_t *dst_block_ids,
+                           size_t n_blocks);
+/* estimated_bytes (src/decoder.rs:273-289). */
+size_t skv_snapshot_bytes(const skv_snapshot *snapshot);
+void skv_snapshot_free(skv_snapshot *snapshot);
+/* snapshot_linear_attn_states / restore (src/metal_backend/linear_attention.rs:3027-3067,
+ * 3163-3198): n device buffers (conv and ssm state of every linear-attention layer)
+ * copied in one launch. Pointers must be 16-byte aligned. */
+int32_t skv_state_snapshot(skv_ctx *ctx, skv_stream stream, const void *const *dev_ptrs,
+                           const size_t *bytes, size_t n, skv_snapshot **out);
+int32_t skv_state_restore(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snapshot,
+                          void *const *dev_ptrs, const size_t *bytes, size_t n);
+
+/* ---- prefix hot cache, host index: BlockHash + BlockAwarePrefixCache -------- */
+
+/* BlockHash::root / for_session / chain (src/serve/cache.rs:10-47). A null or empty key
+ * gives the root; tokens are hashed as u64 little-endian after the previous digest. */
+void skv_hash_root(uint8_t out[32]);
+void skv_hash_for_session(const char *key, size_t key_len, uint8_t out[32]);
+void skv_hash_chain(const uint8_t previous[32], const uint64_t *tokens, size_t n, uint8_t out[32]);
+
+/* PrefixBlockHit (src/serve/cache.rs:50-60) with an opaque payload in place of the state. */
+typedef struct skv_hit {
+    size_t tokens;
+    uint8_t hash[32];
+    uint64_t payload;
+    size_t matched_blocks;
+} skv_hit;
+
+/* with_blocks_per_session / from_runtime_flags (src/serve/cache.rs:83-112); block_tokens 0 -> 1. */
+int32_t skv_prefix_create(size_t block_tokens, size_t capacity, size_t blocks_per_session,
+                          skv_prefix **out);
+int32_t skv_prefix_from_runtime_flags(skv_prefix **out);
+void skv_prefix_destroy(skv_prefix *cache);
+size_t skv_prefix_block_tokens(const skv_prefix *cache);
+size_t skv_prefix_capacity(const skv_prefix *cache);
+size_t skv_prefix_len(const skv_prefix *cache);
+/* estimated_bytes (src/serve/cache.rs:202-204). */
+size_t skv_prefix_bytes(const skv_prefix *cache);
+size_t skv_prefix_session_block_count(const skv_prefix *cache, const uint8_t session[32]);
+/* match_prefix (src/serve/cache.rs:121-151). *found = 1 and *hit filled on a hit;
+ * chain_payloads (optional, chain_cap entries) receives the payload of every matched
+ * block in chain order. */
+int32_t skv_prefix_match(skv_prefix *cache, const uint8_t root[32], const uint64_t *tokens, size_t n,
+                         int32_t *found, skv_hit *hit, uint64_t *chain_payloads, size_t chain_cap);
+/* insert (src/serve/cache.rs:154-193). Payloads that leave the index (an equal key that was
+ * replaced, the session's least recent block, the global least recent block, or the new
+ * payload itself when capacity is 0) are written to `dropped` (at least 4 places) so the
+ * caller can release what they stand for. *bytes_out is insert's return value. */
+int32_t skv_prefix_insert(skv_prefix *cache, const uint8_t session[32], const uint8_t hash[32],
+                          size_t tokens, uint64_t payload, size_t bytes, uint64_t *dropped,
+                          size_t dropped_cap, size_t *n_dropped, size_t *bytes_out);
+/* evict_lru_block (src/serve/cache.rs:196-198). */
+int32_t skv_prefix_evict_lru(skv_prefix *cache, int32_t *found, uint64_t *payload, size_t *bytes);
+/* Entry `index` in recency order (0 = most recent): the tests' view of `cache.entries`. */
+int32_t skv_prefix_entry(const skv_prefix *cache, size_t index, uint8_t session[32], uint8_t hash[32],
+                         size_t *tokens, uint64_t *payload, size_t *bytes);
+
+/* ---- prefix hot cache on the GPU: page pool + index --------------------------- */
+
+/* A pool of `pool_blocks` prefix blocks (each block_tokens/16 page slots holding K and V
+ * of every layer) indexed like BlockAwarePrefixCache. `layers` fixes the shapes the pool
+ * is laid out for; any set of layers with the same shapes can be used afterwards. */
+int32_t skv_hot_create(skv_ctx *ctx, size_t block_tokens, size_t capacity_blocks,
+                       size_t blocks_per_session, size_t pool_blocks, skv_layer *const *layers,
+                       size_t n_layers, skv_hot **out);
+void skv_hot_destroy(skv_hot *hot);
+/* remember_prefix_block (src/serve/state.rs:613-639) for the block of rows
+ * [tokens - block_tokens, tokens): evicts least-recent blocks while the pool is full,
+ * copies the pages (and, if n_states > 0, the recurrent-state buffers) and inserts.
+ * *cached = 0 when nothing was left to evict or the cache is disabled (no error). */
+int32_t skv_hot_remember(skv_hot *hot, skv_stream stream, const uint8_t session[32],
+                         const uint8_t hash[32], size_t tokens, skv_layer *const *layers,
+                         size_t n_layers, const void *const *state_ptrs, const size_t *state_bytes,
+                         size_t n_states, int32_t *cached);
+/* The hit branch of prefill_prompt_state (src/serve/state.rs:574-584): longest cached
+ * chain for `tokens` under `root`, its pages gathered into rows [0, *reused_tokens) of the
+ * layers, the last block's recurrent state copied to state_ptrs, each layer's len set to
+ * *reused_tokens. *reused_tokens = 0 on a miss (layers untouched). */
+int32_t skv_hot_match_restore(skv_hot *hot, skv_stream stream, const uint8_t root[32],
+                              const uint64_t *tokens, size_t n_tokens, skv_layer *const *layers,
+                              size_t n_layers, void *const *state_ptrs, const size_t *state_bytes,
+                              size_t n_states, size_t *reused_tokens, uint8_t hash_out[32]);
+/* evict_prefix_block (src/serve/state.rs:644-646). */
+int32_t skv_hot_evict_lru(skv_hot *hot, int32_t *found, size_t *bytes);
+size_t skv_hot_block_tokens(const skv_hot *hot);
+size_t skv_hot_len(const skv_hot *hot);
+/* prefix_cache_bytes (src/serve/state.rs:640-642). */
+size_t skv_hot_bytes(const skv_hot *hot);
+size_t skv_hot_free_blocks(const skv_hot *hot);
+size_t skv_hot_pool_blocks(const skv_hot *hot);
+size_t skv_hot_block_bytes(const skv_hot *hot);
+uint64_t skv_hot_evictions(const skv_hot *hot);
+uint64_t skv_hot_skipped(const skv_hot *hot);
+int32_t skv_hot_entry(const skv_hot *hot, size_t index, uint8_t session[32], uint8_t hash[32],
+                      size_t *tokens, size_t *bytes);
+
 #ifdef __cplusplus
 }
 #endif

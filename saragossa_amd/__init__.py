@@ -10,7 +10,10 @@ from ._lib import (KvError, DimensionError, ConfigError, DeviceError, lib, lib_p
                    DTYPE_BF16, DTYPE_F32, PAGE_ROWS)
 from .kv import DecodeResidentState, FullAttentionState
 from . import flags
+from .prefix import (BlockHash, BlockAwarePrefixCache, PrefixBlockHit, HotCache, Snapshot,
+                     snapshot_blocks, restore_blocks, state_snapshot, state_restore)
 
 __all__ = ["KvError", "DimensionError", "ConfigError", "DeviceError", "lib", "lib_path",
            "DecodeResidentState", "FullAttentionState", "flags", "DTYPE_BF16", "DTYPE_F32",
-           "PAGE_ROWS"]
+           "PAGE_ROWS", "BlockHash", "BlockAwarePrefixCache", "PrefixBlockHit", "HotCache",
+           "Snapshot", "snapshot_blocks", "restore_blocks", "state_snapshot", "state_restore"]

@@ -86,6 +86,46 @@ SIGNATURES = {
     "skv_decode_step_layers_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_read_rows": (_i32, [_vp, _sz, _sz, _vp, _vp]),
     "skv_gather_device": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp]),
+    "skv_snapshot_blocks": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, C.POINTER(_vp)]),
+    "skv_snapshot_clone": (_i32, [_vp, _vp, _vp, C.POINTER(_vp)]),
+    "skv_restore_blocks": (_i32, [_vp, _vp, _vp, _vp, _sz, _vp, _sz]),
+    "skv_snapshot_bytes": (_sz, [_vp]),
+    "skv_snapshot_free": (None, [_vp]),
+    "skv_state_snapshot": (_i32, [_vp, _vp, _vp, _vp, _sz, C.POINTER(_vp)]),
+    "skv_state_restore": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz]),
+    "skv_hash_root": (None, [_vp]),
+    "skv_hash_for_session": (None, [C.c_char_p, _sz, _vp]),
+    "skv_hash_chain": (None, [_vp, _vp, _sz, _vp]),
+    "skv_prefix_create": (_i32, [_sz, _sz, _sz, C.POINTER(_vp)]),
+    "skv_prefix_from_runtime_flags": (_i32, [C.POINTER(_vp)]),
+    "skv_prefix_destroy": (None, [_vp]),
+    "skv_prefix_block_tokens": (_sz, [_vp]),
+    "skv_prefix_capacity": (_sz, [_vp]),
+    "skv_prefix_len": (_sz, [_vp]),
+    "skv_prefix_bytes": (_sz, [_vp]),
+    "skv_prefix_session_block_count": (_sz, [_vp, _vp]),
+    "skv_prefix_match": (_i32, [_vp, _vp, _vp, _sz, C.POINTER(_i32), _vp, _vp, _sz]),
+    "skv_prefix_insert": (_i32, [_vp, _vp, _vp, _sz, C.c_uint64, _sz, _vp, _sz,
+                                 C.POINTER(_sz), C.POINTER(_sz)]),
+    "skv_prefix_evict_lru": (_i32, [_vp, C.POINTER(_i32), C.POINTER(C.c_uint64), C.POINTER(_sz)]),
+    "skv_prefix_entry": (_i32, [_vp, _sz, _vp, _vp, C.POINTER(_sz), C.POINTER(C.c_uint64),
+                                C.POINTER(_sz)]),
+    "skv_hot_create": (_i32, [_vp, _sz, _sz, _sz, _sz, _vp, _sz, C.POINTER(_vp)]),
+    "skv_hot_destroy": (None, [_vp]),
+    "skv_hot_remember": (_i32, [_vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz,
+                                C.POINTER(_i32)]),
+    "skv_hot_match_restore": (_i32, [_vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz,
+                                     C.POINTER(_sz), _vp]),
+    "skv_hot_evict_lru": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_sz)]),
+    "skv_hot_block_tokens": (_sz, [_vp]),
+    "skv_hot_len": (_sz, [_vp]),
+    "skv_hot_bytes": (_sz, [_vp]),
+    "skv_hot_free_blocks": (_sz, [_vp]),
+    "skv_hot_pool_blocks": (_sz, [_vp]),
+    "skv_hot_block_bytes": (_sz, [_vp]),
+    "skv_hot_evictions": (C.c_uint64, [_vp]),
+    "skv_hot_skipped": (C.c_uint64, [_vp]),
+    "skv_hot_entry": (_i32, [_vp, _sz, _vp, _vp, C.POINTER(_sz), C.POINTER(_sz)]),
 }
 
 

@@ -9,7 +9,7 @@
 #include <string>
 #include <vector>
 
-#include "skv_internal.h"
+#include "layer.h"
 
 namespace skv {
 
@@ -28,37 +28,6 @@ int32_t fail_hip(hipError_t e, const char *what) {
 } // namespace skv
 
 using namespace skv;
-
-struct skv_ctx {
-    int device = 0;
-    hipStream_t stream = nullptr;
-};
-
-struct skv_layer {
-    skv_ctx *ctx = nullptr;
-    Geom g{};
-    size_t capacity = 0;
-    size_t len = 0;
-    size_t window = 0;    // 0 = full cache
-    size_t floor_pos = 0; // ring layers: oldest position still held
-    int n_pages = 0;
-    uint16_t *k_pool = nullptr;
-    uint16_t *v_pool = nullptr;
-    int32_t *table_dev = nullptr;
-    std::vector<int32_t> table;
-    // split-K partials
-    int max_splits = 1;
-    float *part_o = nullptr;
-    float *part_m = nullptr;
-    float *part_l = nullptr;
-    unsigned *counters = nullptr;
-    // staging for the synchronous host entry points
-    float *q_stage = nullptr;   // [q_dim]
-    float *out_stage = nullptr; // [q_dim]
-    float *kv_stage = nullptr;  // [2*kv_dim]
-    float *scores = nullptr;    // plain kernel: [q_heads][capacity], allocated on first use
-    size_t scores_cap = 0;
-};
 
 namespace {
 
@@ -268,7 +237,7 @@ void skv_layer_destroy(skv_layer *L) {
     (void)hipSetDevice(L->ctx->device);
     (void)hipDeviceSynchronize();
     for (void *p : {(void *)L->k_pool, (void *)L->v_pool, (void *)L->table_dev, (void *)L->part_o,
-                    (void *)L->part_m, (void *)L->part_l, (void *)L->counters, (void *)L->q_stage,
+                    (void *)L->part_m, (void *)L->part_l, (void *)L->q_stage,
                     (void *)L->out_stage, (void *)L->kv_stage, (void *)L->scores})
         if (p) (void)hipFree(p);
     delete L;
@@ -328,7 +297,6 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     alloc((void **)&L->part_o, n_part * head_dim * sizeof(float));
     alloc((void **)&L->part_m, n_part * sizeof(float));
     alloc((void **)&L->part_l, n_part * sizeof(float));
-    alloc((void **)&L->counters, kv_heads * sizeof(unsigned));
     alloc((void **)&L->q_stage, q_dim * sizeof(float));
     alloc((void **)&L->out_stage, q_dim * sizeof(float));
     alloc((void **)&L->kv_stage, 2 * kv_dim * sizeof(float));
@@ -336,7 +304,6 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     // query padding; they must hold finite values, so the pools start at zero.
     if (e == hipSuccess) e = hipMemsetAsync(L->k_pool, 0, pool_bytes, ctx->stream);
     if (e == hipSuccess) e = hipMemsetAsync(L->v_pool, 0, pool_bytes, ctx->stream);
-    if (e == hipSuccess) e = hipMemsetAsync(L->counters, 0, kv_heads * sizeof(unsigned), ctx->stream);
     L->table.resize(L->n_pages);
     for (int i = 0; i < L->n_pages; ++i) L->table[i] = i;
     if (e == hipSuccess)

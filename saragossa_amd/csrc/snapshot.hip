@@ -1,0 +1,599 @@
+// Block snapshot / restore of the paged cache, recurrent-state snapshots, and the GPU
+// side of the prefix hot cache (a pool of page slots indexed by the chained block
+// hash with LRU eviction). Stands in for snapshot/copy/restore_prompt_state_metal
+// (src/decoder/generation.rs:2834-2892, 3041-3103), the blits of
+// src/metal_backend/linear_attention.rs:3027-3067, 3163-3198, and the GPU half of
+// remember_prefix_block / prefill_prompt_state (src/serve/state.rs:560-639).
+#include <algorithm>
+#include <cstring>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "layer.h"
+#include "prefix.h"
+
+namespace skv {
+
+// ---- one launch copies up to COPY_MAX_PAGES pages of up to COPY_MAX_LAYERS layers --------
+constexpr int COPY_MAX_LAYERS = 56;
+constexpr int COPY_MAX_PAGES = 128;
+
+struct CopyLayer {
+    uint16_t *k_pool;
+    uint16_t *v_pool;
+    const int32_t *table;
+    uint64_t slot_off;    // byte offset of this layer's K page inside a slot; V follows it
+    uint32_t page_bytes;  // bytes of one K (or V) page of this layer
+    uint32_t ring_pages;  // 0, or the ring's page count (logical page -> page % ring_pages)
+    uint32_t first_page;  // logical pages below this one are skipped (rows a ring no longer holds)
+    uint32_t pad;
+};
+
+struct CopyArgs {
+    CopyLayer layers[COPY_MAX_LAYERS];
+    int32_t layer_page[COPY_MAX_PAGES]; // logical page inside every layer
+    int32_t slot[COPY_MAX_PAGES];       // page slot inside the snapshot storage
+    uint8_t *base;                      // snapshot storage
+    uint64_t slot_bytes;                // one 16-token page across all layers, K and V
+    int n_layers;
+    int n_pages;
+    int to_snapshot; // 1: cache -> storage, 0: storage -> cache
+};
+
+// One workgroup per (page, layer, K|V): a contiguous page_bytes chunk on both sides,
+// 16-byte loads, eight in flight per thread.
+__global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
+    const int chunk = blockIdx.x;
+    const int kv = chunk & 1;
+    const int li = (chunk >> 1) % a.n_layers;
+    const int pi = (chunk >> 1) / a.n_layers;
+    const CopyLayer &L = a.layers[li];
+    const uint32_t lp = (uint32_t)a.layer_page[pi];
+    if (lp < L.first_page) return;
+    const uint32_t tp = L.ring_pages ? lp % L.ring_pages : lp;
+    const int page = L.table[tp];
+    uint8_t *cache = reinterpret_cast<uint8_t *>(kv ? L.v_pool : L.k_pool) + (size_t)page * L.page_bytes;
+    uint8_t *store = a.base + (size_t)a.slot[pi] * a.slot_bytes + L.slot_off + (size_t)kv * L.page_bytes;
+    const uint4 *src = reinterpret_cast<const uint4 *>(a.to_snapshot ? cache : store);
+    uint4 *dst = reinterpret_cast<uint4 *>(a.to_snapshot ? store : cache);
+    const int n16 = (int)(L.page_bytes >> 4);
+    for (int i = threadIdx.x; i < n16; i += 256 * 8) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (i + u * 256 < n16) v[u] = src[i + u * 256];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (i + u * 256 < n16) dst[i + u * 256] = v[u];
+    }
+}
+
+// ---- flat copies of several device buffers in one launch (recurrent state) ----------------
+constexpr int FLAT_MAX = 120;
+struct FlatArgs {
+    const uint8_t *src[FLAT_MAX];
+    uint8_t *dst[FLAT_MAX];
+    uint64_t bytes[FLAT_MAX];
+    int n;
+};
+
+// grid (chunks, buffers): each workgroup strides over its buffer in 32 KiB steps
+__global__ __launch_bounds__(256) void flat_copy_kernel(FlatArgs a) {
+    const int b = blockIdx.y;
+    const uint64_t n = a.bytes[b];
+    const uint64_t n16 = n >> 4;
+    const uint4 *src = reinterpret_cast<const uint4 *>(a.src[b]);
+    uint4 *dst = reinterpret_cast<uint4 *>(a.dst[b]);
+    for (uint64_t i = (uint64_t)blockIdx.x * 2048 + threadIdx.x; i < n16;
+         i += (uint64_t)gridDim.x * 2048) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (i + u * 256 < n16) v[u] = src[i + u * 256];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (i + u * 256 < n16) dst[i + u * 256] = v[u];
+    }
+    if (blockIdx.x == 0) // tail bytes of a buffer whose size is not a multiple of 16
+        for (uint64_t i = (n16 << 4) + threadIdx.x; i < n; i += 256) a.dst[b][i] = a.src[b][i];
+}
+
+static int32_t launch_flat(const void *const *src, void *const *dst, const size_t *bytes, size_t n,
+                           hipStream_t s) {
+    for (size_t first = 0; first < n; first += FLAT_MAX) {
+        FlatArgs a{};
+        a.n = (int)std::min<size_t>(FLAT_MAX, n - first);
+        uint64_t largest = 0;
+        for (int i = 0; i < a.n; ++i) {
+            a.src[i] = (const uint8_t *)src[first + i];
+            a.dst[i] = (uint8_t *)dst[first + i];
+            a.bytes[i] = bytes[first + i];
+            if (((uintptr_t)a.src[i] | (uintptr_t)a.dst[i]) & 15)
+                return fail(SKV_ERR_DEVICE, "copie d'état: pointeur non aligné sur 16 octets");
+            largest = std::max<uint64_t>(largest, a.bytes[i]);
+        }
+        const unsigned chunks = (unsigned)std::min<uint64_t>(std::max<uint64_t>((largest + 32767) / 32768, 1), 1024);
+        hipLaunchKernelGGL(flat_copy_kernel, dim3(chunks, (unsigned)a.n), dim3(256), 0, s, a);
+        SKV_HIP(hipGetLastError());
+    }
+    return SKV_OK;
+}
+
+// Shapes of the layers a storage area was laid out for.
+struct SlotLayout {
+    std::vector<uint32_t> page_bytes; // per layer
+    std::vector<uint64_t> slot_off;
+    uint64_t slot_bytes = 0;
+
+    void build(skv_layer *const *layers, size_t n) {
+        page_bytes.resize(n);
+        slot_off.resize(n);
+        slot_bytes = 0;
+        for (size_t i = 0; i < n; ++i) {
+            page_bytes[i] = (uint32_t)((size_t)layers[i]->g.page_elems * sizeof(uint16_t));
+            slot_off[i] = slot_bytes;
+            slot_bytes += 2ull * page_bytes[i];
+        }
+    }
+    bool matches(skv_layer *const *layers, size_t n) const {
+        if (n != page_bytes.size()) return false;
+        for (size_t i = 0; i < n; ++i)
+            if (page_bytes[i] != (uint32_t)((size_t)layers[i]->g.page_elems * sizeof(uint16_t))) return false;
+        return true;
+    }
+};
+
+// Copies pages between `layers` and the storage at `base`: logical page layer_pages[i] of
+// every layer <-> slot slots[i]. first_page[l] (optional) skips the low pages of layer l.
+static int32_t copy_pages(const SlotLayout &lay, uint8_t *base, skv_layer *const *layers,
+                          size_t n_layers, const int32_t *layer_pages, const int32_t *slots,
+                          size_t n_pages, const uint32_t *first_page, bool to_snapshot,
+                          hipStream_t s) {
+    for (size_t l0 = 0; l0 < n_layers; l0 += COPY_MAX_LAYERS) {
+        const size_t nl = std::min<size_t>(COPY_MAX_LAYERS, n_layers - l0);
+        for (size_t p0 = 0; p0 < n_pages; p0 += COPY_MAX_PAGES) {
+            CopyArgs a{};
+            a.n_layers = (int)nl;
+            a.n_pages = (int)std::min<size_t>(COPY_MAX_PAGES, n_pages - p0);
+            a.base = base;
+            a.slot_bytes = lay.slot_bytes;
+            a.to_snapshot = to_snapshot ? 1 : 0;
+            for (size_t i = 0; i < nl; ++i) {
+                skv_layer *L = layers[l0 + i];
+                CopyLayer &c = a.layers[i];
+                c.k_pool = L->k_pool;
+                c.v_pool = L->v_pool;
+                c.table = L->table_dev;
+                c.slot_off = lay.slot_off[l0 + i];
+                c.page_bytes = lay.page_bytes[l0 + i];
+                c.ring_pages = L->g.ring_rows > 0 ? (uint32_t)L->n_pages : 0;
+                c.first_page = first_page ? first_page[l0 + i] : 0;
+            }
+            for (int i = 0; i < a.n_pages; ++i) {
+                a.layer_page[i] = layer_pages[p0 + i];
+                a.slot[i] = slots[p0 + i];
+            }
+            hipLaunchKernelGGL(page_copy_kernel, dim3((unsigned)(a.n_pages * a.n_layers * 2)), dim3(256),
+                               0, s, a);
+            SKV_HIP(hipGetLastError());
+        }
+    }
+    return SKV_OK;
+}
+
+static int32_t check_layers(skv_ctx *ctx, skv_layer *const *layers, size_t n_layers) {
+    if (!ctx || !layers || n_layers == 0) return fail(SKV_ERR_DEVICE, "snapshot: pointeur nul");
+    for (size_t i = 0; i < n_layers; ++i)
+        if (!layers[i] || layers[i]->ctx != ctx) return fail(SKV_ERR_DEVICE, "snapshot: couche invalide");
+    return SKV_OK;
+}
+
+} // namespace skv
+
+using namespace skv;
+
+struct skv_snapshot {
+    skv_ctx *ctx = nullptr;
+    uint8_t *base = nullptr;
+    size_t bytes = 0;
+    // block snapshots
+    SlotLayout layout;
+    size_t n_pages = 0;
+    // state snapshots
+    std::vector<size_t> sizes;   // bytes of each buffer
+    std::vector<size_t> offsets; // 256-byte aligned offsets inside `base`
+};
+
+static hipStream_t as_stream(skv_stream s) { return reinterpret_cast<hipStream_t>(s); }
+
+struct HotEntry {
+    std::vector<int32_t> slots;  // one per 16-token page of the block
+    skv_snapshot *state = nullptr; // recurrent state at the block boundary, or null
+    size_t bytes = 0;
+};
+
+struct skv_hot {
+    skv_ctx *ctx = nullptr;
+    PrefixIndex *index = nullptr;
+    SlotLayout layout;
+    size_t pages_per_block = 0;
+    size_t pool_slots = 0;
+    uint8_t *pool = nullptr;
+    std::vector<int32_t> free_slots;
+    std::unordered_map<uint64_t, HotEntry> entries;
+    uint64_t next_id = 1;
+    // counters (x-saragossa-reused-prefix-tokens accounting and eviction log, serve/state.rs:59-80, 263-266)
+    uint64_t evictions = 0;
+    uint64_t skipped = 0;
+};
+
+static void hot_release(skv_hot *h, uint64_t id) {
+    auto it = h->entries.find(id);
+    if (it == h->entries.end()) return;
+    for (int32_t s : it->second.slots) h->free_slots.push_back(s);
+    if (it->second.state) skv_snapshot_free(it->second.state);
+    h->entries.erase(it);
+}
+
+extern "C" {
+
+// ---- block snapshots ----------------------------------------------------------------------
+int32_t skv_snapshot_blocks(skv_ctx *ctx, skv_stream stream, skv_layer *const *layers,
+                            size_t n_layers, const size_t *block_ids, size_t n_blocks,
+                            skv_snapshot **out) {
+    if (!out) return fail(SKV_ERR_DEVICE, "snapshot_blocks: out nul");
+    *out = nullptr;
+    int32_t rc = check_layers(ctx, layers, n_layers);
+    if (rc) return rc;
+    if (n_blocks && !block_ids) return fail(SKV_ERR_DEVICE, "snapshot_blocks: block_ids nul");
+    std::vector<int32_t> pages(n_blocks), slots(n_blocks);
+    for (size_t i = 0; i < n_blocks; ++i) {
+        for (size_t l = 0; l < n_layers; ++l) {
+            const skv_layer *L = layers[l];
+            if (block_ids[i] * 16 >= L->len)
+                return fail(SKV_ERR_DIMENSION, "snapshot_blocks: bloc " + std::to_string(block_ids[i]) +
+                                                   " au-delà de len " + std::to_string(L->len));
+            if (L->g.ring_rows > 0 && block_ids[i] * 16 < L->floor_pos)
+                return fail(SKV_ERR_DIMENSION, "snapshot_blocks: bloc déjà évincé de l'anneau");
+        }
+        pages[i] = (int32_t)block_ids[i];
+        slots[i] = (int32_t)i;
+    }
+    SKV_HIP(hipSetDevice(ctx->device));
+    skv_snapshot *snap = new skv_snapshot();
+    snap->ctx = ctx;
+    snap->layout.build(layers, n_layers);
+    snap->n_pages = n_blocks;
+    snap->bytes = n_blocks * snap->layout.slot_bytes;
+    if (snap->bytes) {
+        hipError_t e = hipMalloc((void **)&snap->base, snap->bytes);
+        if (e != hipSuccess) {
+            delete snap;
+            return fail_hip(e, "snapshot_blocks: allocation");
+        }
+        rc = copy_pages(snap->layout, snap->base, layers, n_layers, pages.data(), slots.data(),
+                        n_blocks, nullptr, true, as_stream(stream));
+        if (rc) {
+            skv_snapshot_free(snap);
+            return rc;
+        }
+    }
+    *out = snap;
+    return SKV_OK;
+}
+
+int32_t skv_restore_blocks(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snap,
+                           skv_layer *const *layers, size_t n_layers, const size_t *dst_block_ids,
+                           size_t n_blocks) {
+    if (!snap) return fail(SKV_ERR_DEVICE, "restore_blocks: snapshot nul");
+    int32_t rc = check_layers(ctx, layers, n_layers);
+    if (rc) return rc;
+    if (!snap->sizes.empty()) return fail(SKV_ERR_DEVICE, "restore_blocks: snapshot d'état, pas de blocs");
+    if (!snap->layout.matches(layers, n_layers))
+        return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=" + std::to_string(snap->layout.page_bytes.size()) +
+                                           " couches=" + std::to_string(n_layers) + " ou formes différentes");
+    if (n_blocks != snap->n_pages)
+        return fail(SKV_ERR_DIMENSION, "restore_blocks: " + std::to_string(n_blocks) + " blocs, snapshot de " +
+                                           std::to_string(snap->n_pages));
+    std::vector<int32_t> pages(n_blocks), slots(n_blocks);
+    for (size_t i = 0; i < n_blocks; ++i) {
+        for (size_t l = 0; l < n_layers; ++l) {
+            const skv_layer *L = layers[l];
+            const size_t cap_pages = L->g.ring_rows > 0 ? (L->capacity + 15) / 16 : (size_t)L->n_pages;
+            if (dst_block_ids[i] >= cap_pages)
+                return fail(SKV_ERR_DIMENSION, "restore_blocks: bloc " + std::to_string(dst_block_ids[i]) +
+                                                   " > capacité");
+        }
+        pages[i] = (int32_t)dst_block_ids[i];
+        slots[i] = (int32_t)i;
+    }
+    if (n_blocks == 0) return SKV_OK;
+    SKV_HIP(hipSetDevice(ctx->device));
+    return copy_pages(snap->layout, snap->base, layers, n_layers, pages.data(), slots.data(), n_blocks,
+                      nullptr, false, as_stream(stream));
+}
+
+int32_t skv_snapshot_clone(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snap,
+                           skv_snapshot **out) {
+    if (!ctx || !snap || !out) return fail(SKV_ERR_DEVICE, "snapshot_clone: pointeur nul");
+    *out = nullptr;
+    SKV_HIP(hipSetDevice(ctx->device));
+    skv_snapshot *c = new skv_snapshot(*snap);
+    c->base = nullptr;
+    if (c->bytes) {
+        hipError_t e = hipMalloc((void **)&c->base, c->bytes);
+        if (e != hipSuccess) {
+            delete c;
+            return fail_hip(e, "snapshot_clone: allocation");
+        }
+        const void *src = snap->base;
+        void *dst = c->base;
+        int32_t rc = launch_flat(&src, &dst, &c->bytes, 1, as_stream(stream));
+        if (rc) {
+            skv_snapshot_free(c);
+            return rc;
+        }
+    }
+    *out = c;
+    return SKV_OK;
+}
+
+size_t skv_snapshot_bytes(const skv_snapshot *snap) { return snap ? snap->bytes : 0; }
+
+void skv_snapshot_free(skv_snapshot *snap) {
+    if (!snap) return;
+    if (snap->base) {
+        (void)hipSetDevice(snap->ctx->device);
+        (void)hipDeviceSynchronize(); // copies that read or write it may still be queued
+        (void)hipFree(snap->base);
+    }
+    delete snap;
+}
+
+// ---- recurrent-state snapshots ---------------------------------------------------------------
+int32_t skv_state_snapshot(skv_ctx *ctx, skv_stream stream, const void *const *dev_ptrs,
+                           const size_t *bytes, size_t n, skv_snapshot **out) {
+    if (!ctx || !out || (n && (!dev_ptrs || !bytes))) return fail(SKV_ERR_DEVICE, "state_snapshot: pointeur nul");
+    *out = nullptr;
+    SKV_HIP(hipSetDevice(ctx->device));
+    skv_snapshot *snap = new skv_snapshot();
+    snap->ctx = ctx;
+    size_t total = 0;
+    for (size_t i = 0; i < n; ++i) {
+        if (!dev_ptrs[i]) {
+            delete snap;
+            return fail(SKV_ERR_DEVICE, "state_snapshot: pointeur nul");
+        }
+        snap->sizes.push_back(bytes[i]);
+        snap->offsets.push_back(total);
+        total += (bytes[i] + 255) / 256 * 256;
+    }
+    snap->bytes = total;
+    if (total) {
+        hipError_t e = hipMalloc((void **)&snap->base, total);
+        if (e != hipSuccess) {
+            delete snap;
+            return fail_hip(e, "state_snapshot: allocation");
+        }
+        std::vector<void *> dst(n);
+        for (size_t i = 0; i < n; ++i) dst[i] = snap->base + snap->offsets[i];
+        int32_t rc = launch_flat(dev_ptrs, dst.data(), bytes, n, as_stream(stream));
+        if (rc) {
+            skv_snapshot_free(snap);
+            return rc;
+        }
+    }
+    if (n == 0) snap->sizes.clear();
+    *out = snap;
+    return SKV_OK;
+}
+
+int32_t skv_state_restore(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snap,
+                          void *const *dev_ptrs, const size_t *bytes, size_t n) {
+    if (!ctx || !snap || (n && (!dev_ptrs || !bytes))) return fail(SKV_ERR_DEVICE, "state_restore: pointeur nul");
+    if (n != snap->sizes.size())
+        return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=" + std::to_string(snap->sizes.size()) +
+                                           " couches=" + std::to_string(n));
+    for (size_t i = 0; i < n; ++i)
+        if (bytes[i] != snap->sizes[i])
+            return fail(SKV_ERR_DIMENSION, "state_restore: taille du tampon " + std::to_string(i) + " différente");
+    if (n == 0) return SKV_OK;
+    SKV_HIP(hipSetDevice(ctx->device));
+    std::vector<const void *> src(n);
+    for (size_t i = 0; i < n; ++i) src[i] = snap->base + snap->offsets[i];
+    return launch_flat(src.data(), dev_ptrs, bytes, n, as_stream(stream));
+}
+
+// ---- the hot cache: page pool + index ----------------------------------------------------------
+int32_t skv_hot_create(skv_ctx *ctx, size_t block_tokens, size_t capacity_blocks,
+                       size_t blocks_per_session, size_t pool_blocks, skv_layer *const *layers,
+                       size_t n_layers, skv_hot **out) {
+    if (!out) return fail(SKV_ERR_DEVICE, "hot_create: out nul");
+    *out = nullptr;
+    int32_t rc = check_layers(ctx, layers, n_layers);
+    if (rc) return rc;
+    if (block_tokens == 0 || block_tokens % 16 != 0)
+        return fail(SKV_ERR_CONFIG, "prefix-cache GPU: block_tokens doit être un multiple de 16");
+    SKV_HIP(hipSetDevice(ctx->device));
+    skv_hot *h = new skv_hot();
+    h->ctx = ctx;
+    h->index = new PrefixIndex(block_tokens, capacity_blocks, blocks_per_session);
+    h->layout.build(layers, n_layers);
+    h->pages_per_block = block_tokens / 16;
+    h->pool_slots = pool_blocks * h->pages_per_block;
+    const size_t bytes = h->pool_slots * h->layout.slot_bytes;
+    if (bytes) {
+        hipError_t e = hipMalloc((void **)&h->pool, bytes);
+        if (e != hipSuccess) {
+            delete h->index;
+            delete h;
+            return fail_hip(e, "hot_create: allocation du pool");
+        }
+    }
+    h->free_slots.reserve(h->pool_slots);
+    for (size_t i = h->pool_slots; i-- > 0;) h->free_slots.push_back((int32_t)i);
+    *out = h;
+    return SKV_OK;
+}
+
+void skv_hot_destroy(skv_hot *h) {
+    if (!h) return;
+    (void)hipSetDevice(h->ctx->device);
+    (void)hipDeviceSynchronize();
+    for (auto &kv : h->entries)
+        if (kv.second.state) skv_snapshot_free(kv.second.state);
+    if (h->pool) (void)hipFree(h->pool);
+    delete h->index;
+    delete h;
+}
+
+size_t skv_hot_block_tokens(const skv_hot *h) { return h ? h->index->block_tokens() : 0; }
+size_t skv_hot_len(const skv_hot *h) { return h ? h->index->len() : 0; }
+size_t skv_hot_bytes(const skv_hot *h) { return h ? h->index->bytes() : 0; }
+size_t skv_hot_free_blocks(const skv_hot *h) { return h ? h->free_slots.size() / h->pages_per_block : 0; }
+size_t skv_hot_pool_blocks(const skv_hot *h) { return h ? h->pool_slots / h->pages_per_block : 0; }
+size_t skv_hot_block_bytes(const skv_hot *h) { return h ? h->pages_per_block * h->layout.slot_bytes : 0; }
+uint64_t skv_hot_evictions(const skv_hot *h) { return h ? h->evictions : 0; }
+uint64_t skv_hot_skipped(const skv_hot *h) { return h ? h->skipped : 0; }
+
+int32_t skv_hot_entry(const skv_hot *h, size_t index, uint8_t session[32], uint8_t hash[32],
+                      size_t *tokens, size_t *bytes) {
+    if (!h) return fail(SKV_ERR_DEVICE, "hot_entry: pointeur nul");
+    if (!h->index->entry(index, session, hash, tokens, nullptr, bytes))
+        return fail(SKV_ERR_DIMENSION, "hot_entry: index " + std::to_string(index) + " hors plage");
+    return SKV_OK;
+}
+
+int32_t skv_hot_evict_lru(skv_hot *h, int32_t *found, size_t *bytes) {
+    if (!h || !found) return fail(SKV_ERR_DEVICE, "hot_evict_lru: pointeur nul");
+    uint64_t id = 0;
+    const bool ok = h->index->evict_lru(&id, bytes);
+    *found = ok ? 1 : 0;
+    if (ok) {
+        hot_release(h, id);
+        ++h->evictions;
+    }
+    return SKV_OK;
+}
+
+// remember_prefix_block (src/serve/state.rs:613-639): snapshot the block that ends at
+// `tokens`, evict least-recent blocks while the pool has no room, then insert. When nothing
+// is left to evict the block is skipped without an error (*cached = 0).
+int32_t skv_hot_remember(skv_hot *h, skv_stream stream, const uint8_t session[32],
+                         const uint8_t hash[32], size_t tokens, skv_layer *const *layers,
+                         size_t n_layers, const void *const *state_ptrs, const size_t *state_bytes,
+                         size_t n_states, int32_t *cached) {
+    if (!h || !session || !hash || !cached) return fail(SKV_ERR_DEVICE, "hot_remember: pointeur nul");
+    *cached = 0;
+    int32_t rc = check_layers(h->ctx, layers, n_layers);
+    if (rc) return rc;
+    if (!h->layout.matches(layers, n_layers))
+        return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: les couches n'ont pas la forme du pool");
+    const size_t bt = h->index->block_tokens();
+    if (tokens < bt || tokens % bt != 0)
+        return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: tokens=" + std::to_string(tokens) +
+                                           " n'est pas une frontière de bloc");
+    for (size_t l = 0; l < n_layers; ++l) {
+        if (layers[l]->len < tokens)
+            return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: couche plus courte que la frontière");
+        if (layers[l]->g.ring_rows > 0 && tokens - bt < layers[l]->floor_pos)
+            return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: bloc déjà évincé de l'anneau");
+    }
+    if (h->index->capacity() == 0) return SKV_OK; // insert() of a disabled cache stores nothing
+    SKV_HIP(hipSetDevice(h->ctx->device));
+    while (h->free_slots.size() < h->pages_per_block) {
+        uint64_t id = 0;
+        if (!h->index->evict_lru(&id, nullptr)) {
+            ++h->skipped;
+            return SKV_OK; // nothing left to evict: skip caching, no error
+        }
+        hot_release(h, id);
+        ++h->evictions;
+    }
+    HotEntry e;
+    std::vector<int32_t> pages(h->pages_per_block);
+    for (size_t i = 0; i < h->pages_per_block; ++i) {
+        e.slots.push_back(h->free_slots.back());
+        h->free_slots.pop_back();
+        pages[i] = (int32_t)((tokens - bt) / 16 + i);
+    }
+    rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), e.slots.data(),
+                    h->pages_per_block, nullptr, true, as_stream(stream));
+    if (!rc && n_states)
+        rc = skv_state_snapshot(h->ctx, stream, state_ptrs, state_bytes, n_states, &e.state);
+    if (rc) {
+        for (int32_t s : e.slots) h->free_slots.push_back(s);
+        return rc;
+    }
+    e.bytes = h->pages_per_block * h->layout.slot_bytes + (e.state ? e.state->bytes : 0);
+    const uint64_t id = h->next_id++;
+    const size_t nbytes = e.bytes;
+    h->entries.emplace(id, std::move(e));
+    std::vector<uint64_t> dropped;
+    h->index->insert(session, hash, tokens, id, nbytes, &dropped);
+    for (uint64_t d : dropped) {
+        if (d != id) ++h->evictions;
+        hot_release(h, d);
+    }
+    *cached = h->entries.count(id) ? 1 : 0;
+    return SKV_OK;
+}
+
+// The hit branch of prefill_prompt_state (src/serve/state.rs:574-584): longest chain of
+// cached blocks for `tokens`, every matched block's pages copied into the layers' rows
+// [0, reused), the recurrent state of the last matched block copied out, len = reused.
+int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[32],
+                              const uint64_t *tokens, size_t n_tokens, skv_layer *const *layers,
+                              size_t n_layers, void *const *state_ptrs, const size_t *state_bytes,
+                              size_t n_states, size_t *reused_tokens, uint8_t hash_out[32]) {
+    if (!h || !root || !reused_tokens || (n_tokens && !tokens))
+        return fail(SKV_ERR_DEVICE, "hot_match_restore: pointeur nul");
+    *reused_tokens = 0;
+    int32_t rc = check_layers(h->ctx, layers, n_layers);
+    if (rc) return rc;
+    if (!h->layout.matches(layers, n_layers))
+        return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: les couches n'ont pas la forme du pool");
+    PrefixHit hit{};
+    std::vector<uint64_t> chain;
+    if (!h->index->match(root, tokens, n_tokens, &hit, &chain)) return SKV_OK;
+    const size_t reused = hit.tokens;
+    for (size_t l = 0; l < n_layers; ++l)
+        if (reused > layers[l]->capacity)
+            return fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(reused) + " > capacité " +
+                                               std::to_string(layers[l]->capacity));
+    SKV_HIP(hipSetDevice(h->ctx->device));
+    std::vector<int32_t> pages, slots;
+    for (size_t b = 0; b < chain.size(); ++b) {
+        const HotEntry &e = h->entries.at(chain[b]);
+        for (size_t i = 0; i < e.slots.size(); ++i) {
+            pages.push_back((int32_t)(b * h->pages_per_block + i));
+            slots.push_back(e.slots[i]);
+        }
+    }
+    std::vector<uint32_t> first_page(n_layers, 0);
+    for (size_t l = 0; l < n_layers; ++l) {
+        const skv_layer *L = layers[l];
+        if (L->g.ring_rows > 0 && reused > (size_t)L->g.ring_rows)
+            first_page[l] = (uint32_t)((reused - (size_t)L->g.ring_rows + 15) / 16);
+    }
+    rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(), pages.size(),
+                    first_page.data(), false, as_stream(stream));
+    if (rc) return rc;
+    const HotEntry &last = h->entries.at(chain.back());
+    if (n_states) {
+        if (!last.state) return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=0 couches=" + std::to_string(n_states));
+        rc = skv_state_restore(h->ctx, stream, last.state, state_ptrs, state_bytes, n_states);
+        if (rc) return rc;
+    }
+    for (size_t l = 0; l < n_layers; ++l) {
+        skv_layer *L = layers[l];
+        L->len = reused;
+        L->floor_pos = (size_t)first_page[l] * 16;
+    }
+    *reused_tokens = reused;
+    if (hash_out) std::memcpy(hash_out, hit.hash, 32);
+    return SKV_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,236 @@
+"""Prefix hot cache on the GPU: block snapshot / restore / gather through the hash index
+with LRU eviction, bit-exact against re-derived contents and, for the control flow,
+against the restatement of the reference's serve algorithm (src/serve/state.rs:560-639)."""
+import numpy as np
+import pytest
+
+import oracle
+import saragossa_amd as skv
+from oracle import prefix_cache as pc
+from saragossa_amd import BlockHash
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def make_layers(state, n_layers, capacity, dims=(32, 8, 128), seed=0, window=0):
+    rng = np.random.default_rng(seed)
+    layers = []
+    for _ in range(n_layers):
+        kv = state.full_attention_bf16(capacity, *dims, window=window)
+        kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+        layers.append(kv)
+    return layers
+
+
+def rows_for(layer, positions, tokens, kv_dim, seed=3):
+    """K/V rows as a deterministic function of (layer, position, the token prefix), so that any
+    restored row can be re-derived and a wrong block is detected."""
+    tokens = np.asarray(tokens, dtype=np.uint64)
+    prefix = np.cumsum(tokens * np.uint64(2654435761) + np.uint64(97), dtype=np.uint64)
+    out_k = np.empty((len(positions), kv_dim), dtype=np.float32)
+    out_v = np.empty_like(out_k)
+    cols = np.arange(kv_dim, dtype=np.uint64)
+    for i, p in enumerate(positions):
+        base = (prefix[p] ^ np.uint64(layer * 7919 + seed * 104729 + p * 31)) & np.uint64(0xFFFFFFFF)
+        x = (base * np.uint64(1103515245) + cols * np.uint64(12345)) & np.uint64(0xFFFFFF)
+        out_k[i] = (x.astype(np.float32) / np.float32(2 ** 23) - np.float32(1.0))
+        out_v[i] = -out_k[i] * np.float32(0.75) + np.float32(0.125)
+    return out_k, out_v
+
+
+def fill(layers, first, last, tokens, kv_dim):
+    for li, kv in enumerate(layers):
+        k, v = rows_for(li, range(first, last), tokens, kv_dim)
+        kd, vd = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+        kv.encode_append_batch(_stream(), kd.data_ptr(), vd.data_ptr(), last - first)
+        torch.cuda.synchronize()
+
+
+def check_contents(layers, n, tokens, kv_dim):
+    for li, kv in enumerate(layers):
+        assert kv.len() == n
+        k, v = rows_for(li, range(n), tokens, kv_dim)
+        gk, gv = kv.read_rows()
+        assert np.array_equal(gk, oracle.f32_to_bf16_bits(k)), f"layer {li} K"
+        assert np.array_equal(gv, oracle.f32_to_bf16_bits(v)), f"layer {li} V"
+
+
+def test_snapshot_restore_roundtrip_and_clone_independence(state):
+    # the decoder/tests.rs:297-346 pattern: restoring from a copy leaves the entry pristine
+    dims, kv_dim, n = (16, 2, 256), 512, 16 * 6
+    tokens = list(range(n))
+    a = make_layers(state, 3, n, dims, seed=1)
+    fill(a, 0, n, tokens, kv_dim)
+    snap = skv.snapshot_blocks(state, a, [1, 2, 4], stream=_stream())
+    assert snap.estimated_bytes() == 3 * 3 * 2 * 16 * kv_dim * 2
+    copy = snap.clone(stream=_stream())
+    torch.cuda.synchronize()
+    # overwrite the source blocks, then restore into another set of layers at other block ids
+    b = make_layers(state, 3, n, dims, seed=2)
+    fill(b, 0, n, [t + 1000 for t in tokens], kv_dim)
+    skv.restore_blocks(state, copy, b, [0, 5, 3], stream=_stream())
+    torch.cuda.synchronize()
+    for li in range(3):
+        ak, av = a[li].read_rows()
+        bk, bv = b[li].read_rows()
+        for src, dst in [(1, 0), (2, 5), (4, 3)]:
+            assert np.array_equal(bk[dst * 16:dst * 16 + 16], ak[src * 16:src * 16 + 16])
+            assert np.array_equal(bv[dst * 16:dst * 16 + 16], av[src * 16:src * 16 + 16])
+        k_other, _ = rows_for(li, range(16, 32), [t + 1000 for t in tokens], kv_dim)
+        assert np.array_equal(bk[16:32], oracle.f32_to_bf16_bits(k_other))   # untouched block
+    # the original snapshot still restores the original bytes after the copy was used
+    a[0].truncate(0)
+    fill([a[0]], 0, n, [7] * n, kv_dim)
+    for kv in a[1:]:
+        kv.truncate(0)
+        kv.truncate(n)
+    a[0].truncate(n)
+    skv.restore_blocks(state, snap, a, [1, 2, 4], stream=_stream())
+    k0, _ = rows_for(0, range(16, 48), tokens, kv_dim)
+    gk, _ = a[0].read_rows(16, 32)
+    assert np.array_equal(gk, oracle.f32_to_bf16_bits(k0))
+    # shape / count mismatches are Dimension errors (src/decoder/generation.rs:3086-3092)
+    with pytest.raises(skv.DimensionError):
+        skv.restore_blocks(state, snap, a[:2], [1, 2, 4])
+    with pytest.raises(skv.DimensionError):
+        skv.restore_blocks(state, snap, a, [1, 2])
+    with pytest.raises(skv.DimensionError):
+        skv.snapshot_blocks(state, a, [6])       # beyond len
+    other = make_layers(state, 3, n, (8, 2, 64))
+    with pytest.raises(skv.DimensionError):
+        skv.restore_blocks(state, snap, other, [1, 2, 4])
+
+
+def test_linear_attn_state_snapshot_restore_roundtrip(state):
+    # src/metal_backend/tests/linear_attention.rs:12-...: conv (96 KiB) + ssm (2 MiB) per layer
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    sizes = [3 * 8192 * 4, 32 * 128 * 128 * 4] * 4 + [100]        # an odd-sized buffer too
+    bufs = [torch.randint(0, 255, (s,), dtype=torch.uint8, device="cuda", generator=gen)
+            for s in sizes]
+    want = [b.clone() for b in bufs]
+    snap = skv.state_snapshot(state, [b.data_ptr() for b in bufs], sizes, stream=_stream())
+    assert snap.estimated_bytes() >= sum(sizes)
+    for b in bufs:
+        b.zero_()
+    skv.state_restore(state, snap, [b.data_ptr() for b in bufs], sizes, stream=_stream())
+    torch.cuda.synchronize()
+    for b, w in zip(bufs, want):
+        assert torch.equal(b, w)
+    with pytest.raises(skv.DimensionError):
+        skv.state_restore(state, snap, [b.data_ptr() for b in bufs[:-1]], sizes[:-1])
+
+
+class SimDecoder(pc.PromptDecoder):
+    """The oracle side of the multi-turn run: state = number of tokens consumed."""
+
+    class S:
+        def __init__(self, n): self.n = n
+        def clone(self): return SimDecoder.S(self.n)
+
+    def prefill_uncached(self, tokens): return SimDecoder.S(len(tokens))
+    def extend(self, state, tokens): state.n += len(tokens)
+
+
+@pytest.mark.parametrize("dims,n_layers,bt,prefix,pool_frac", [
+    ((32, 8, 128), 4, 16, 256, 0.6),     # BASELINE config 3 shapes, scaled down
+    ((16, 2, 256), 2, 32, 128, 0.5),     # two pages per hash block
+])
+def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims, n_layers, bt,
+                                                                     prefix, pool_frac):
+    kv_dim = dims[1] * dims[2]
+    rng = np.random.default_rng(33)
+    n_sessions, vocab = 6, 151936
+    shared = [int(t) for t in rng.integers(0, vocab, size=prefix)]
+    hist = [[int(t) for t in rng.integers(0, vocab, size=rng.integers(bt, 4 * bt))]
+            for _ in range(n_sessions)]
+    turns = [[int(t) for t in rng.integers(0, vocab, size=2 * bt + 5)] for _ in range(n_sessions)]
+    # distinct blocks the traffic produces: the shared prefix once, then each session's own
+    demand = len(shared) // bt + sum((len(shared) + len(h) + len(t)) // bt - len(shared) // bt
+                                     for h, t in zip(hist, turns))
+    pool_blocks = int(demand * pool_frac)
+    cap = max(len(shared + h + t) for h, t in zip(hist, turns)) + 16
+    proto = make_layers(state, n_layers, 16, dims)
+    hot = skv.HotCache(state, bt, 10 ** 6, pool_blocks, proto)
+    assert hot.pool_blocks() == pool_blocks and hot.block_bytes() == n_layers * 2 * bt * kv_dim * 2
+    # oracle run of the same traffic: byte budget = pool size
+    ocache = pc.BlockAwarePrefixCache(bt, 10 ** 6, state_bytes=lambda s, m: 1)
+    over = lambda extra: len(ocache.entries) + extra > pool_blocks
+    odec = SimDecoder()
+
+    def run_turn(session_key, tokens):
+        layers = make_layers(state, n_layers, cap, dims, seed=len(tokens))
+        root = BlockHash.for_session(session_key)
+        reused, h = hot.match_restore(root, tokens, layers, stream=_stream())
+        _, want_reused = pc.prefill_prompt_state(ocache, odec, tokens, session_key, over)
+        assert reused == want_reused
+        h = h or root
+        consumed = reused
+        while consumed + bt <= len(tokens) // bt * bt:
+            fill(layers, consumed, consumed + bt, tokens, kv_dim)
+            h = BlockHash.chain(h, tokens[consumed:consumed + bt])
+            consumed += bt
+            hot.remember_prefix_block(root, h, consumed, layers, stream=_stream())
+        if consumed < len(tokens):
+            fill(layers, consumed, len(tokens), tokens, kv_dim)
+        torch.cuda.synchronize()
+        check_contents(layers, len(tokens), tokens, kv_dim)
+        assert [(e["hash"], e["tokens"]) for e in hot.entries] == \
+               [(e.hash, e.tokens) for e in ocache.entries]
+        for kv in layers:
+            kv.close()
+        return reused
+
+    total_reused = 0
+    for s in range(n_sessions):                 # first contact: shared prefix + history
+        total_reused += run_turn(None, shared + hist[s])
+    for s in range(n_sessions):                 # second turn: everything so far + the new turn
+        total_reused += run_turn(None, shared + hist[s] + turns[s])
+    assert total_reused > 0 and hot.evictions() > 0
+    assert len(hot) <= pool_blocks and hot.free_blocks() == pool_blocks - len(hot)
+    # sessions are isolated by their root
+    assert run_turn("agent-a", shared + hist[0]) == 0
+    # drain: evict_lru_block returns the bytes of each victim, then None
+    n = len(hot)
+    got = [hot.evict_lru_block() for _ in range(n)]
+    assert got == [hot.block_bytes()] * n and hot.evict_lru_block() is None
+    assert hot.free_blocks() == pool_blocks
+    hot.close()
+
+
+def test_hot_cache_with_recurrent_state_and_skip_when_nothing_to_evict(state):
+    dims, kv_dim, bt = (16, 2, 256), 512, 16
+    layers = make_layers(state, 2, 64, dims)
+    tokens = list(range(100, 148))
+    fill(layers, 0, 48, tokens, kv_dim)
+    ssm = torch.arange(4096, dtype=torch.float32, device="cuda")
+    hot = skv.HotCache(state, bt, 8, 2, layers)
+    root = BlockHash.root()
+    h1 = BlockHash.chain(root, tokens[:16])
+    h2 = BlockHash.chain(h1, tokens[16:32])
+    assert hot.remember_prefix_block(root, h1, 16, layers, [ssm.data_ptr()], [ssm.numel() * 4])
+    ssm += 1.0
+    assert hot.remember_prefix_block(root, h2, 32, layers, [ssm.data_ptr()], [ssm.numel() * 4])
+    assert hot.estimated_bytes() == 2 * (hot.block_bytes() + ssm.numel() * 4)
+    fresh = make_layers(state, 2, 64, dims, seed=9)
+    out = torch.zeros_like(ssm)
+    reused, h = hot.match_restore(root, tokens, fresh, [out.data_ptr()], [out.numel() * 4])
+    torch.cuda.synchronize()
+    assert reused == 32 and h == h2
+    assert torch.equal(out, torch.arange(4096, dtype=torch.float32, device="cuda") + 1.0)
+    check_contents(fresh, 32, tokens, kv_dim)
+    # a disabled cache (capacity 0) and a pool with no room and nothing to evict both skip silently
+    off = skv.HotCache(state, bt, 0, 2, layers)
+    assert not off.remember_prefix_block(root, h1, 16, layers)
+    tiny = skv.HotCache(state, bt, 8, 0, layers)
+    assert not tiny.remember_prefix_block(root, h1, 16, layers) and tiny.skipped() == 1
+    with pytest.raises(skv.DimensionError):
+        hot.remember_prefix_block(root, h1, 24, layers)        # not a block boundary
+    with pytest.raises(skv.DimensionError):
+        hot.remember_prefix_block(root, h1, 64, layers)        # beyond len
+    with pytest.raises(skv.ConfigError):
+        skv.HotCache(state, 24, 8, 2, layers)                  # not a multiple of the page size
