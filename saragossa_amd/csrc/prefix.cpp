@@ -7,6 +7,7 @@
 // are O(1); every observable order (what a match leaves behind, which entry a
 // per-session or global eviction removes) is the reference's.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <iterator>
 #include <list>
@@ -15,6 +16,10 @@
 #include <vector>
 
 #include "prefix.h"
+
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
 
 namespace skv {
 
@@ -43,7 +48,63 @@ void Sha256::reset() {
     fill_ = 0;
 }
 
+#if defined(__x86_64__)
+// One or more 64-byte blocks with the x86 SHA extensions (sha256rnds2 / sha256msg1 /
+// sha256msg2), used when the host CPU has them. Same function as the portable code below;
+// both are checked against FIPS 180-4 vectors.
+__attribute__((target("sha,sse4.1,ssse3"))) static void sha256_blocks_ni(uint32_t state[8],
+                                                                         const uint8_t *data) {
+    const __m128i mask = _mm_set_epi64x(0x0c0d0e0f08090a0bLL, 0x0405060700010203LL);
+    __m128i tmp = _mm_loadu_si128(reinterpret_cast<const __m128i *>(&state[0]));
+    __m128i st1 = _mm_loadu_si128(reinterpret_cast<const __m128i *>(&state[4]));
+    tmp = _mm_shuffle_epi32(tmp, 0xB1);              // CDAB
+    st1 = _mm_shuffle_epi32(st1, 0x1B);              // EFGH
+    __m128i st0 = _mm_alignr_epi8(tmp, st1, 8);      // ABEF
+    st1 = _mm_blend_epi16(st1, tmp, 0xF0);           // CDGH
+    const __m128i abef = st0, cdgh = st1;
+    __m128i m[4];
+    for (int i = 0; i < 4; ++i)
+        m[i] = _mm_shuffle_epi8(_mm_loadu_si128(reinterpret_cast<const __m128i *>(data + 16 * i)), mask);
+    for (int i = 0; i < 16; ++i) {
+        const int cur = i & 3;
+        __m128i msg = _mm_add_epi32(m[cur], _mm_loadu_si128(reinterpret_cast<const __m128i *>(&K256[4 * i])));
+        st1 = _mm_sha256rnds2_epu32(st1, st0, msg);
+        if (i >= 3 && i < 15) { // message words of the group after next
+            const __m128i t = _mm_alignr_epi8(m[cur], m[(cur + 3) & 3], 4);
+            m[(cur + 1) & 3] = _mm_sha256msg2_epu32(_mm_add_epi32(m[(cur + 1) & 3], t), m[cur]);
+        }
+        msg = _mm_shuffle_epi32(msg, 0x0E);
+        st0 = _mm_sha256rnds2_epu32(st0, st1, msg);
+        if (i >= 1 && i < 13) m[(cur + 3) & 3] = _mm_sha256msg1_epu32(m[(cur + 3) & 3], m[cur]);
+    }
+    st0 = _mm_add_epi32(st0, abef);
+    st1 = _mm_add_epi32(st1, cdgh);
+    tmp = _mm_shuffle_epi32(st0, 0x1B);              // FEBA
+    st1 = _mm_shuffle_epi32(st1, 0xB1);              // DCHG
+    st0 = _mm_blend_epi16(tmp, st1, 0xF0);           // DCBA
+    st1 = _mm_alignr_epi8(st1, tmp, 8);              // HGFE
+    _mm_storeu_si128(reinterpret_cast<__m128i *>(&state[0]), st0);
+    _mm_storeu_si128(reinterpret_cast<__m128i *>(&state[4]), st1);
+}
+
+static bool have_sha_ni() {
+    static const bool ok = [] {
+        const char *force = std::getenv("SKV_SHA_PORTABLE");
+        if (force && force[0] == '1') return false;
+        return __builtin_cpu_supports("sha") && __builtin_cpu_supports("sse4.1") &&
+               __builtin_cpu_supports("ssse3");
+    }();
+    return ok;
+}
+#endif
+
 void Sha256::block(const uint8_t *p) {
+#if defined(__x86_64__)
+    if (have_sha_ni()) {
+        sha256_blocks_ni(h_, p);
+        return;
+    }
+#endif
     uint32_t w[64];
     for (int i = 0; i < 16; ++i)
         w[i] = ((uint32_t)p[4 * i] << 24) | ((uint32_t)p[4 * i + 1] << 16) |
@@ -111,11 +172,15 @@ void Sha256::finish(uint8_t out[32]) {
 void hash_chain(const uint8_t prev[32], const uint64_t *tokens, size_t n, uint8_t out[32]) {
     Sha256 h;
     h.update(prev, 32);
+#if defined(__BYTE_ORDER__) && __BYTE_ORDER__ == __ORDER_LITTLE_ENDIAN__
+    h.update(tokens, n * sizeof(uint64_t)); // already u64 little-endian in memory
+#else
     for (size_t i = 0; i < n; ++i) {
         uint8_t le[8];
         for (int b = 0; b < 8; ++b) le[b] = (uint8_t)(tokens[i] >> (8 * b));
         h.update(le, 8);
     }
+#endif
     h.finish(out);
 }
 
@@ -185,31 +250,50 @@ size_t PrefixIndex::session_block_count(const uint8_t session[32]) const {
 bool PrefixIndex::match(const uint8_t root[32], const uint64_t *tokens, size_t n, PrefixHit *hit,
                         std::vector<uint64_t> *chain) {
     if (chain) chain->clear();
-    if (capacity_ == 0) return false;
-    uint8_t previous[32];
-    std::memcpy(previous, root, 32);
-    bool found = false;
+    Walk w;
+    match_start(&w, root);
+    return match_more(&w, root, tokens, n, (size_t)-1, hit, chain) > 0;
+}
+
+void PrefixIndex::match_start(Walk *w, const uint8_t root[32]) const {
+    std::memcpy(w->previous, root, 32);
+    w->index = 0;
+    w->alive = capacity_ != 0;
+}
+
+size_t PrefixIndex::match_more(Walk *w, const uint8_t root[32], const uint64_t *tokens, size_t n,
+                               size_t max_blocks, PrefixHit *hit, std::vector<uint64_t> *chain) {
+    if (!w->alive) return 0;
     const size_t blocks = n / block_tokens_; // chunks_exact
-    for (size_t index = 0; index < blocks; ++index) {
+    size_t matched = 0;
+    while (matched < max_blocks) {
+        if (w->index >= blocks) {
+            w->alive = false;
+            break;
+        }
         Impl::Key key;
         std::memcpy(key.session, root, 32);
-        hash_chain(previous, tokens + index * block_tokens_, block_tokens_, key.hash);
-        key.tokens = (index + 1) * block_tokens_;
+        hash_chain(w->previous, tokens + w->index * block_tokens_, block_tokens_, key.hash);
+        key.tokens = (w->index + 1) * block_tokens_;
         auto it = impl_->map.find(key);
-        if (it == impl_->map.end()) break;
+        if (it == impl_->map.end()) {
+            w->alive = false;
+            break;
+        }
         impl_->lru.splice(impl_->lru.begin(), impl_->lru, it->second); // remove + insert(0)
         const Impl::Node &node = *it->second;
         if (hit) {
             hit->tokens = node.key.tokens;
             std::memcpy(hit->hash, node.key.hash, 32);
             hit->payload = node.payload;
-            hit->matched_blocks = index + 1;
+            hit->matched_blocks = w->index + 1;
         }
         if (chain) chain->push_back(node.payload);
-        std::memcpy(previous, key.hash, 32);
-        found = true;
+        std::memcpy(w->previous, key.hash, 32);
+        ++w->index;
+        ++matched;
     }
-    return found;
+    return matched;
 }
 
 // insert (src/serve/cache.rs:154-193). Payloads that leave the index (a replaced equal

@@ -50,6 +50,17 @@ class PrefixIndex {
     size_t session_block_count(const uint8_t session[32]) const;
     bool match(const uint8_t root[32], const uint64_t *tokens, size_t n, PrefixHit *hit,
                std::vector<uint64_t> *chain);
+    // The same walk in steps, so that a caller can act on the first matched blocks while
+    // the rest of the chain is still being hashed. match_more() appends to `chain` and
+    // returns how many further blocks matched (fewer than max_blocks: the walk is over).
+    struct Walk {
+        uint8_t previous[32];
+        size_t index = 0;
+        bool alive = true;
+    };
+    void match_start(Walk *w, const uint8_t root[32]) const;
+    size_t match_more(Walk *w, const uint8_t root[32], const uint64_t *tokens, size_t n,
+                      size_t max_blocks, PrefixHit *hit, std::vector<uint64_t> *chain);
     size_t insert(const uint8_t session[32], const uint8_t hash[32], size_t tokens,
                   uint64_t payload, size_t bytes, std::vector<uint64_t> *dropped);
     bool evict_lru(uint64_t *payload, size_t *bytes);

@@ -41,6 +41,24 @@ struct CopyArgs {
     int to_snapshot; // 1: cache -> storage, 0: storage -> cache
 };
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Streams n16 16-byte words from src to dst: eight independent loads in flight per thread,
+// then eight stores, all non-temporal (the data is touched once; keeping it out of the
+// caches leaves them to the attention kernels and measurably raises copy bandwidth).
+__device__ __forceinline__ void copy_stream(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst,
+                                            long n16, long first, long stride) {
+    long i = first;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], dst + i + u * stride);
+    }
+    for (; i < n16; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
 // One workgroup per (page, layer, K|V): a contiguous page_bytes chunk on both sides,
 // 16-byte loads, eight in flight per thread.
 __global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
@@ -55,18 +73,9 @@ __global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
     const int page = L.table[tp];
     uint8_t *cache = reinterpret_cast<uint8_t *>(kv ? L.v_pool : L.k_pool) + (size_t)page * L.page_bytes;
     uint8_t *store = a.base + (size_t)a.slot[pi] * a.slot_bytes + L.slot_off + (size_t)kv * L.page_bytes;
-    const uint4 *src = reinterpret_cast<const uint4 *>(a.to_snapshot ? cache : store);
-    uint4 *dst = reinterpret_cast<uint4 *>(a.to_snapshot ? store : cache);
-    const int n16 = (int)(L.page_bytes >> 4);
-    for (int i = threadIdx.x; i < n16; i += 256 * 8) {
-        uint4 v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (i + u * 256 < n16) v[u] = src[i + u * 256];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (i + u * 256 < n16) dst[i + u * 256] = v[u];
-    }
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(a.to_snapshot ? cache : store);
+    u32x4 *dst = reinterpret_cast<u32x4 *>(a.to_snapshot ? store : cache);
+    copy_stream(src, dst, (long)(L.page_bytes >> 4), threadIdx.x, 256);
 }
 
 // ---- flat copies of several device buffers in one launch (recurrent state) ----------------
@@ -78,25 +87,15 @@ struct FlatArgs {
     int n;
 };
 
-// grid (chunks, buffers): each workgroup strides over its buffer in 32 KiB steps
+// grid (chunks, buffers): the workgroups of a buffer stride over it together
 __global__ __launch_bounds__(256) void flat_copy_kernel(FlatArgs a) {
     const int b = blockIdx.y;
     const uint64_t n = a.bytes[b];
-    const uint64_t n16 = n >> 4;
-    const uint4 *src = reinterpret_cast<const uint4 *>(a.src[b]);
-    uint4 *dst = reinterpret_cast<uint4 *>(a.dst[b]);
-    for (uint64_t i = (uint64_t)blockIdx.x * 2048 + threadIdx.x; i < n16;
-         i += (uint64_t)gridDim.x * 2048) {
-        uint4 v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (i + u * 256 < n16) v[u] = src[i + u * 256];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (i + u * 256 < n16) dst[i + u * 256] = v[u];
-    }
+    const long n16 = (long)(n >> 4);
+    copy_stream(reinterpret_cast<const u32x4 *>(a.src[b]), reinterpret_cast<u32x4 *>(a.dst[b]), n16,
+                (long)blockIdx.x * 256 + threadIdx.x, (long)gridDim.x * 256);
     if (blockIdx.x == 0) // tail bytes of a buffer whose size is not a multiple of 16
-        for (uint64_t i = (n16 << 4) + threadIdx.x; i < n; i += 256) a.dst[b][i] = a.src[b][i];
+        for (uint64_t i = ((uint64_t)n16 << 4) + threadIdx.x; i < n; i += 256) a.dst[b][i] = a.src[b][i];
 }
 
 static int32_t launch_flat(const void *const *src, void *const *dst, const size_t *bytes, size_t n,
@@ -554,32 +553,69 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
     if (rc) return rc;
     if (!h->layout.matches(layers, n_layers))
         return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: les couches n'ont pas la forme du pool");
+    size_t min_capacity = (size_t)-1;
+    bool any_ring = false;
+    for (size_t l = 0; l < n_layers; ++l) {
+        min_capacity = std::min(min_capacity, layers[l]->capacity);
+        any_ring = any_ring || layers[l]->g.ring_rows > 0;
+    }
+    SKV_HIP(hipSetDevice(h->ctx->device));
+    // The chain of SHA-256 digests is inherently serial on the host (about 0.3 us per
+    // block); the walk therefore proceeds in growing batches and the pages of each batch
+    // are put in flight while the next one is being hashed. Ring layers need the final
+    // length to know which rows still fit, so for them the walk finishes first.
     PrefixHit hit{};
     std::vector<uint64_t> chain;
-    if (!h->index->match(root, tokens, n_tokens, &hit, &chain)) return SKV_OK;
-    const size_t reused = hit.tokens;
-    for (size_t l = 0; l < n_layers; ++l)
-        if (reused > layers[l]->capacity)
-            return fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(reused) + " > capacité " +
-                                               std::to_string(layers[l]->capacity));
-    SKV_HIP(hipSetDevice(h->ctx->device));
+    PrefixIndex::Walk walk;
+    h->index->match_start(&walk, root);
     std::vector<int32_t> pages, slots;
-    for (size_t b = 0; b < chain.size(); ++b) {
-        const HotEntry &e = h->entries.at(chain[b]);
-        for (size_t i = 0; i < e.slots.size(); ++i) {
-            pages.push_back((int32_t)(b * h->pages_per_block + i));
-            slots.push_back(e.slots[i]);
+    size_t done_blocks = 0; // blocks whose copies have been queued
+    size_t batch = any_ring ? (size_t)-1 : 16;
+    const size_t bt = h->index->block_tokens();
+    for (;;) {
+        const size_t got = h->index->match_more(&walk, root, tokens, n_tokens, batch, &hit, &chain);
+        if (chain.size() * bt > min_capacity)
+            return fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(chain.size() * bt) +
+                                               " > capacité " + std::to_string(min_capacity));
+        if (got == 0) break;
+        if (!any_ring) {
+            pages.clear();
+            slots.clear();
+            for (size_t b = done_blocks; b < chain.size(); ++b) {
+                const HotEntry &e = h->entries.at(chain[b]);
+                for (size_t i = 0; i < e.slots.size(); ++i) {
+                    pages.push_back((int32_t)(b * h->pages_per_block + i));
+                    slots.push_back(e.slots[i]);
+                }
+            }
+            rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(),
+                            pages.size(), nullptr, false, as_stream(stream));
+            if (rc) return rc;
+            done_blocks = chain.size();
+            batch = std::min<size_t>(batch * 2, COPY_MAX_PAGES);
         }
+        if (!walk.alive) break;
     }
+    if (chain.empty()) return SKV_OK;
+    const size_t reused = hit.tokens;
     std::vector<uint32_t> first_page(n_layers, 0);
-    for (size_t l = 0; l < n_layers; ++l) {
-        const skv_layer *L = layers[l];
-        if (L->g.ring_rows > 0 && reused > (size_t)L->g.ring_rows)
-            first_page[l] = (uint32_t)((reused - (size_t)L->g.ring_rows + 15) / 16);
+    if (any_ring) {
+        for (size_t b = 0; b < chain.size(); ++b) {
+            const HotEntry &e = h->entries.at(chain[b]);
+            for (size_t i = 0; i < e.slots.size(); ++i) {
+                pages.push_back((int32_t)(b * h->pages_per_block + i));
+                slots.push_back(e.slots[i]);
+            }
+        }
+        for (size_t l = 0; l < n_layers; ++l) {
+            const skv_layer *L = layers[l];
+            if (L->g.ring_rows > 0 && reused > (size_t)L->g.ring_rows)
+                first_page[l] = (uint32_t)((reused - (size_t)L->g.ring_rows + 15) / 16);
+        }
+        rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(), pages.size(),
+                        first_page.data(), false, as_stream(stream));
+        if (rc) return rc;
     }
-    rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(), pages.size(),
-                    first_page.data(), false, as_stream(stream));
-    if (rc) return rc;
     const HotEntry &last = h->entries.at(chain.back());
     if (n_states) {
         if (!last.state) return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=0 couches=" + std::to_string(n_states));
