@@ -154,6 +154,19 @@ int32_t skv_decode_step_device(skv_layer *layer, skv_stream stream, const void *
                                size_t k_off, const void *v_dev, size_t v_off, const float *q_dev,
                                float *out_dev);
 
+/* Chunked prefill over the cache: appends n_rows rows (k_dev, v_dev: [n_rows, kv_dim] f32)
+ * and computes, for every new row i, attention of q_dev[i] over rows 0..len_before+i through
+ * the layer's sliding window: cached_attention_prefill_rows
+ * (src/decoder/attention_ops.rs:976-1017) as one launch on the matrix cores instead of
+ * the reference's per-row loop (src/decode_resident/layers.rs:1113-1118). out_dev is
+ * [n_rows, q_dim] f32. */
+int32_t skv_prefill_chunk_device(skv_layer *layer, skv_stream stream, const float *q_dev,
+                                 const void *k_dev, const void *v_dev, size_t n_rows,
+                                 float *out_dev);
+/* Same with host buffers; synchronous. */
+int32_t skv_prefill_chunk_host(skv_layer *layer, const float *q, const float *k, const float *v,
+                               size_t n_rows, float *out);
+
 /* The KV path of one token over several layers: for each layer i, append
  * k_dev[i]/v_dev[i] (kv_dim f32 each) then attention of q_dev[i] into out_dev[i].
  * It is the per-layer loop of enqueue_decode_token_resident

@@ -43,7 +43,13 @@ int decode_max_splits() { return DEC_MAX_SPLITS; }
 //
 // At the end every wavefront writes its (o, m, l) to LDS and the whole workgroup
 // reduces them column-parallel: with one split that is the final context, otherwise a
-// partial per query head for the merge kernel.
+// partial per query slot for the merge kernel.
+//
+// The same kernel serves chunked prefill over the cache: with n_queries > 1 the query
+// slots are (query row, head of the group) pairs, 16 per workgroup (grid z), and slot
+// (i, g) attends positions up to len - n_queries + i, the causal limit of the i-th new
+// row (the per-row loop of cached_attention_prefill_rows,
+// src/decoder/attention_ops.rs:976-1017, as one launch).
 // ------------------------------------------------------------------------------------
 template <int KK>
 __device__ __forceinline__ void load_k(uint4 (&k)[KK], const DecodeArgs &a, int page, int kvh,
@@ -76,7 +82,23 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     const int j = lane >> 4;
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
+    const int tile = blockIdx.z;
     const int G = g.gqa;
+    const int C = a.n_queries;
+    const int n_slots = C * G;
+    const int rows = min(16, n_slots - tile * 16); // query slots of this workgroup
+    // this lane's query slot in the B and D operand layouts
+    const int my_slot = min(tile * 16 + n, n_slots - 1);
+    const int my_q = my_slot / G;
+    const int my_limit = a.len - C + my_q; // last position the slot attends
+    const int my_ws = a.window > 0 ? max(a.window_start, my_limit + 1 - a.window) : a.window_start;
+    // extremes over the workgroup's slots
+    const int qrow_lo = (tile * 16) / G;
+    const int qrow_hi = (tile * 16 + rows - 1) / G;
+    const int lim_lo = a.len - C + qrow_lo;
+    const int lim_hi = a.len - C + qrow_hi;
+    const int ws_lo = a.window > 0 ? max(a.window_start, lim_lo + 1 - a.window) : a.window_start;
+    const int ws_hi = a.window > 0 ? max(a.window_start, lim_hi + 1 - a.window) : a.window_start;
 
     extern __shared__ __attribute__((aligned(16))) uint4 smem[];
     uint4 *q_hi = smem;
@@ -84,8 +106,11 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     uint16_t *new_k = reinterpret_cast<uint16_t *>(smem + 2 * KK * 64); // [P] appended row
     uint16_t *new_v = new_k + P;
 
-    const int pb0 = a.page_first + (int)(((long)split * a.n_pages) / a.splits);
-    const int pb1 = a.page_first + (int)(((long)(split + 1) * a.n_pages) / a.splits);
+    // pages this workgroup's slots can see, divided among the splits
+    const int page_lo = g.ring_rows > 0 ? 0 : ws_lo >> 4;
+    const int page_hi = g.ring_rows > 0 ? a.n_pages : (lim_hi >> 4) + 1;
+    const int pb0 = page_lo + (int)(((long)split * (page_hi - page_lo)) / a.splits);
+    const int pb1 = page_lo + (int)(((long)(split + 1) * (page_hi - page_lo)) / a.splits);
     // this wavefront walks pages pb0 + wave + it * WAVES, it = 0 .. n_it-1
     const int n_it = pb1 - pb0 > wave ? (pb1 - pb0 - wave + WAVES - 1) / WAVES : 0;
 
@@ -95,7 +120,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     // back from memory in this launch.
     const int pb_new = a.new_slot >> 4;
     const int r_new = a.new_slot & 15;
-    const bool appends = a.k_new != nullptr && pb_new >= pb0 && pb_new < pb1;
+    const bool appends = a.k_new != nullptr && C == 1 && pb_new >= pb0 && pb_new < pb1;
     if (appends) {
         const int page = a.table[pb_new];
         const long tile = (long)page * g.page_elems + (long)kvh * g.tile_elems;
@@ -132,8 +157,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
         const int idx = min(tid + u * THREADS, KK * 64 - 1);
         const int kk = idx >> 6;
         const int jj = (idx >> 4) & 3;
-        const int qn = min(idx & 15, G - 1);
-        const float *qrow = a.q + (long)(kvh * G + qn) * g.head_dim;
+        const int qs = min(tile * 16 + (idx & 15), n_slots - 1);
+        const float *qrow = a.q + ((long)(qs / G) * g.q_heads + kvh * G + qs % G) * g.head_dim;
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[u][e] = qrow[min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
     }
@@ -149,7 +174,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
         if (idx < KK * 64) {
             const int kk = idx >> 6;
             const int jj = (idx >> 4) & 3;
-            const bool row_ok = (idx & 15) < G;
+            const bool row_ok = (idx & 15) < rows;
             uint32_t hi[4], lo[4];
 #pragma unroll
             for (int e2 = 0; e2 < 4; ++e2) {
@@ -197,8 +222,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
         // Only pages that touch the window start, the end of the cache or (ring layers) any
         // page at all can hold keys outside [window_start, len).
         const int first_slot = pb * 16;
-        const bool interior = g.ring_rows == 0 && first_slot >= a.window_start &&
-                              first_slot + 16 <= a.len;
+        const bool interior = g.ring_rows == 0 && first_slot >= ws_hi && first_slot + 16 <= lim_lo + 1;
         if (!interior) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -206,7 +230,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
                 int pos = slot;
                 if (g.ring_rows > 0)
                     pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
-                const bool ok = pos >= a.window_start && pos < a.len;
+                const bool ok = pos >= my_ws && pos <= my_limit;
                 s[i] = ok ? s[i] : -INFINITY;
             }
         }
@@ -308,38 +332,39 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
 
     // ---- all wavefronts publish (o, m, l); the workgroup reduces them column-parallel -------
     __syncthreads(); // the staged queries are no longer needed: the LDS is reused
-    float *xo = reinterpret_cast<float *>(smem);        // [WAVES][G][OSTRIDE]
-    float *xm = xo + WAVES * G * OSTRIDE;               // [WAVES][G]
-    float *xl = xm + WAVES * G;                         // [WAVES][G]
-    if (n < G) {
-        float *dst = xo + (wave * G + n) * OSTRIDE + j * 4;
+    float *xo = reinterpret_cast<float *>(smem);        // [WAVES][rows][OSTRIDE]
+    float *xm = xo + WAVES * rows * OSTRIDE;            // [WAVES][rows]
+    float *xl = xm + WAVES * rows;                      // [WAVES][rows]
+    if (n < rows) {
+        float *dst = xo + (wave * rows + n) * OSTRIDE + j * 4;
 #pragma unroll
         for (int t = 0; t < NT; ++t) *reinterpret_cast<float4_t *>(dst + t * 16) = o[t];
         if (j == 0) {
-            xm[wave * G + n] = m_run;
-            xl[wave * G + n] = l_run;
+            xm[wave * rows + n] = m_run;
+            xl[wave * rows + n] = l_run;
         }
     }
     __syncthreads();
-    for (int idx = tid; idx < G * P; idx += THREADS) {
+    for (int idx = tid; idx < rows * P; idx += THREADS) {
         const int row = idx / P;
         const int col = idx - row * P;
         float mx = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, xm[w * G + row]);
+        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, xm[w * rows + row]);
         const float m_safe = mx == -INFINITY ? 0.0f : mx;
         float acc = 0.0f, lsum = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            const float wgt = fast_exp2(xm[w * G + row] - m_safe);
-            acc += wgt * xo[(w * G + row) * OSTRIDE + col];
-            lsum += wgt * xl[w * G + row];
+            const float wgt = fast_exp2(xm[w * rows + row] - m_safe);
+            acc += wgt * xo[(w * rows + row) * OSTRIDE + col];
+            lsum += wgt * xl[w * rows + row];
         }
         if (col < g.head_dim) {
+            const int slot = tile * 16 + row;
             if (a.splits == 1) {
-                a.out[(long)(kvh * G + row) * g.head_dim + col] = acc / lsum;
+                a.out[((long)(slot / G) * g.q_heads + kvh * G + slot % G) * g.head_dim + col] = acc / lsum;
             } else {
-                const long pidx = ((long)kvh * a.splits + split) * G + row;
+                const long pidx = ((long)kvh * a.splits + split) * n_slots + slot;
                 a.part_o[pidx * g.head_dim + col] = acc;
                 if (col == 0) {
                     a.part_m[pidx] = mx;
@@ -361,18 +386,19 @@ constexpr int MERGE_PER_LANE = DEC_MAX_SPLITS / 16;
 
 __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
     const Geom g = a.g;
-    const int h = blockIdx.x;
-    const int kvh = h / g.gqa;
-    const int gq = h - kvh * g.gqa;
+    const int n_slots = a.n_queries * g.gqa;
+    const int kvh = blockIdx.x / n_slots;
+    const int slot = blockIdx.x - kvh * n_slots;
+    const long h = (long)(slot / g.gqa) * g.q_heads + kvh * g.gqa + slot % g.gqa; // output row
     const int tid = threadIdx.x;
     const int c = tid & 15;
-    const int col = min(blockIdx.y * 16 + c, g.head_dim - 1);
+    const int col = min((int)blockIdx.y * 16 + c, g.head_dim - 1);
     const int sl = tid >> 4;
     __shared__ float red_m[16];
     __shared__ float red_l[16];
     __shared__ float acc_x[16][17];
-    const long base = ((long)kvh * a.splits) * g.gqa + gq;
-    const long ostride = (long)g.gqa * g.head_dim;
+    const long base = ((long)kvh * a.splits) * n_slots + slot;
+    const long ostride = (long)n_slots * g.head_dim;
     const float *po = a.part_o + base * g.head_dim + col;
     float ov[MERGE_PER_LANE], mv[MERGE_PER_LANE], lv[MERGE_PER_LANE];
 #pragma unroll
@@ -380,8 +406,8 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
         const int s = sl + 16 * i;
         const bool ok = s < a.splits;
         const int sc = ok ? s : 0;
-        mv[i] = a.part_m[base + (long)sc * g.gqa];
-        lv[i] = a.part_l[base + (long)sc * g.gqa];
+        mv[i] = a.part_m[base + (long)sc * n_slots];
+        lv[i] = a.part_l[base + (long)sc * n_slots];
         ov[i] = po[(long)sc * ostride];
         if (!ok) {
             mv[i] = -INFINITY;
@@ -414,7 +440,7 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
             t += acc_x[i][c];
             l += red_l[i];
         }
-        a.out[(long)h * g.head_dim + col] = t / l;
+        a.out[h * g.head_dim + col] = t / l;
     }
 }
 
@@ -422,7 +448,9 @@ template <int P, int WAVES>
 static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
     constexpr int KK = P / 32;
     const size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
-    const size_t xchg = ((size_t)WAVES * a.g.gqa * (P + 4) + 2 * WAVES * a.g.gqa) * sizeof(float);
+    const int n_slots = a.n_queries * a.g.gqa;
+    const int rows = n_slots < 16 ? n_slots : 16;
+    const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
     const size_t lds = stage > xchg ? stage : xchg;
     static bool attr_set = false; // per instantiation
     if (!attr_set) {
@@ -432,7 +460,7 @@ static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads);
+    dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
     hipLaunchKernelGGL((decode_split_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
@@ -448,7 +476,7 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     default: break;
     }
     if (e != hipSuccess || a.splits == 1) return e;
-    dim3 mgrid((unsigned)a.g.q_heads, (unsigned)((a.g.head_dim + 15) / 16));
+    dim3 mgrid((unsigned)(a.g.kv_heads * a.n_queries * a.g.gqa), (unsigned)((a.g.head_dim + 15) / 16));
     hipLaunchKernelGGL(decode_merge_kernel, mgrid, dim3(256), 0, s, a);
     return hipGetLastError();
 }

@@ -10,6 +10,8 @@ using skv::Geom;
 struct skv_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
+    void *mq_scratch = nullptr; // split-K partials of multi-query launches, grown on demand
+    size_t mq_bytes = 0;
 };
 
 struct skv_layer {

@@ -92,13 +92,16 @@ bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L-
 
 // k_new / v_new non-null: the row at position len-1 has not been written yet and the
 // attention kernel appends it itself (the host bookkeeping has already advanced).
+// n_queries > 1: chunked prefill over the cache; the last n_queries rows are the new ones
+// and query i attends positions up to len - n_queries + i, each through the layer's
+// sliding window. The matrix-core kernel only.
 int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float *out_dev,
                          size_t window_start, const float *k_new = nullptr,
-                         const float *v_new = nullptr) {
+                         const float *v_new = nullptr, size_t n_queries = 1) {
     int32_t rc = check_window(L, window_start);
     if (rc) return rc;
     const Geom &g = L->g;
-    const bool use_flash = uses_flash(L);
+    const bool use_flash = uses_flash(L) || n_queries > 1;
     if (!use_flash) {
         const size_t need = (size_t)g.q_heads * L->capacity;
         if (L->scores_cap < need) {
@@ -135,6 +138,8 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     a.part_m = L->part_m;
     a.part_l = L->part_l;
     a.len = (int)L->len;
+    a.n_queries = (int)n_queries;
+    a.window = n_queries > 1 ? (int)L->window : 0; // decode callers pass window_start themselves
     a.window_start = (int)window_start;
     if (g.ring_rows > 0) {
         a.page_first = 0;
@@ -147,6 +152,29 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     }
     a.waves = choose_waves(L);
     a.splits = choose_splits(L, a.n_pages, L->len - window_start, a.waves);
+    if (n_queries > 1) {
+        // every 16 query slots are a workgroup of their own: split the context only while
+        // that leaves compute units idle, and keep the partials in the context's scratch
+        const size_t tiles = (n_queries * (size_t)g.gqa + 15) / 16 * (size_t)g.kv_heads;
+        const size_t want = std::max<size_t>(256 / tiles, 1);
+        a.splits = (int)std::min<size_t>((size_t)a.splits, want);
+        if (a.splits > 1) {
+            const size_t n_part = (size_t)g.kv_heads * a.splits * n_queries * g.gqa;
+            const size_t need = n_part * ((size_t)g.head_dim + 2) * sizeof(float);
+            skv_ctx *c = L->ctx;
+            if (c->mq_bytes < need) {
+                SKV_HIP(hipDeviceSynchronize());
+                if (c->mq_scratch) SKV_HIP(hipFree(c->mq_scratch));
+                c->mq_scratch = nullptr;
+                c->mq_bytes = 0;
+                SKV_HIP(hipMalloc(&c->mq_scratch, need));
+                c->mq_bytes = need;
+            }
+            a.part_o = reinterpret_cast<float *>(c->mq_scratch);
+            a.part_m = a.part_o + n_part * g.head_dim;
+            a.part_l = a.part_m + n_part;
+        }
+    }
     // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
     // 575); log2(e) moves the softmax to base 2.
     a.qscale = (1.0f / std::sqrt((float)g.head_dim)) * 1.4426950408889634f;
@@ -222,7 +250,8 @@ int32_t skv_ctx_create(int32_t device, skv_ctx **out) {
 void skv_ctx_destroy(skv_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
-    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipDeviceSynchronize();
+    if (ctx->mq_scratch) (void)hipFree(ctx->mq_scratch);
     delete ctx;
 }
 
@@ -484,6 +513,73 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
                                   reinterpret_cast<const float *>((const char *)v_dev + v_off));
     if (rc) L->len -= 1;
     return rc;
+}
+
+int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q_dev,
+                                 const void *k_dev, const void *v_dev, size_t n_rows,
+                                 float *out_dev) {
+    if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "prefill chunk: pointeur nul");
+    if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "attention batch cached shapes: seq == 0");
+    if (L->g.P > 256) return fail(SKV_ERR_CONFIG, "prefill sur cache: head_dim > 256 non supporté");
+    if (L->len + n_rows > L->capacity)
+        return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
+                                           std::to_string(L->capacity) + " atteinte (overflow)");
+    const size_t kv_dim = skv_kv_dim(L), q_dim = (size_t)L->g.q_heads * L->g.head_dim;
+    // A ring that holds exactly its window cannot take several new rows before the first of
+    // them has been attended: the rows it would overwrite are still inside that query's
+    // window. Such layers advance in steps the ring can hold.
+    size_t step = std::min<size_t>(n_rows, 4096);
+    if (L->g.ring_rows > 0) {
+        const size_t room = (size_t)L->g.ring_rows >= L->window ? (size_t)L->g.ring_rows - L->window + 1 : 1;
+        step = std::min(step, room);
+    }
+    const float *q = q_dev, *k = (const float *)k_dev, *v = (const float *)v_dev;
+    float *out = out_dev;
+    for (size_t done = 0; done < n_rows; done += step) {
+        const size_t c = std::min(step, n_rows - done);
+        int32_t rc = encode_append(L, as_stream(stream), k, v, c);
+        if (rc) return rc;
+        const size_t ws_base = L->g.ring_rows > 0 ? L->floor_pos : 0;
+        const size_t first_ws = std::max(ws_base, skv_window_start(L->len - c, L->window));
+        if (c == 1) {
+            rc = encode_attention(L, as_stream(stream), q, out, first_ws);
+        } else {
+            rc = encode_attention(L, as_stream(stream), q, out, ws_base, nullptr, nullptr, c);
+        }
+        if (rc) return rc;
+        q += c * q_dim;
+        k += c * kv_dim;
+        v += c * kv_dim;
+        out += c * q_dim;
+    }
+    return SKV_OK;
+}
+
+int32_t skv_prefill_chunk_host(skv_layer *L, const float *q, const float *k, const float *v,
+                               size_t n_rows, float *out) {
+    if (!L || !q || !k || !v || !out) return fail(SKV_ERR_DEVICE, "prefill chunk: pointeur nul");
+    if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "attention batch cached shapes: seq == 0");
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    const size_t kv_dim = skv_kv_dim(L), q_dim = (size_t)L->g.q_heads * L->g.head_dim;
+    const size_t qb = n_rows * q_dim * sizeof(float), kb = n_rows * kv_dim * sizeof(float);
+    char *buf = nullptr;
+    SKV_HIP(hipMalloc((void **)&buf, 2 * qb + 2 * kb));
+    float *qd = (float *)buf, *od = (float *)(buf + qb), *kd = (float *)(buf + 2 * qb),
+          *vd = (float *)(buf + 2 * qb + kb);
+    hipStream_t s = L->ctx->stream;
+    hipError_t e = hipMemcpyAsync(qd, q, qb, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(kd, k, kb, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(vd, v, kb, hipMemcpyHostToDevice, s);
+    int32_t rc = SKV_OK;
+    if (e == hipSuccess) rc = skv_prefill_chunk_device(L, s, qd, kd, vd, n_rows, od);
+    if (e == hipSuccess && !rc) e = hipMemcpyAsync(out, od, qb, hipMemcpyDeviceToHost, s);
+    hipError_t e2 = hipStreamSynchronize(s);
+    (void)hipFree(buf);
+    if (e != hipSuccess) return fail_hip(e, "prefill chunk: copie");
+    if (rc) return rc;
+    if (e2 != hipSuccess) return fail_hip(e2, "prefill chunk: synchronisation");
+    return SKV_OK;
 }
 
 int32_t skv_decode_step_layers_device(skv_layer *const *layers, size_t n_layers, skv_stream stream,

@@ -84,16 +84,18 @@ struct GatherArgs {
 };
 
 struct DecodeArgs {
-    const float *q;  // [q_heads*head_dim] f32
-    float *out;      // [q_heads*head_dim] f32
+    const float *q;  // [n_queries][q_heads*head_dim] f32
+    float *out;      // [n_queries][q_heads*head_dim] f32
     const uint16_t *k_pool;
     const uint16_t *v_pool;
     const int32_t *table;
-    float *part_o;   // [kv_heads][splits][gqa][head_dim]
-    float *part_m;   // [kv_heads][splits][gqa]   (log2 domain)
-    float *part_l;   // [kv_heads][splits][gqa]
+    float *part_o;   // [kv_heads][splits][n_queries*gqa][head_dim]
+    float *part_m;   // [kv_heads][splits][n_queries*gqa]   (log2 domain)
+    float *part_l;   // [kv_heads][splits][n_queries*gqa]
     int len;          // rows valid: positions 0..len
-    int window_start; // first position attended
+    int n_queries;    // 1 = decode; C = chunked prefill, query i attends positions <= len-C+i
+    int window;       // sliding window applied per query (0 = none)
+    int window_start; // first position attended (lower bound for every query)
     int ring_base;    // ring layers: (len-1) - (len-1) % ring_rows
     int ring_t;       // ring layers: (len-1) % ring_rows
     int page_first;   // first logical page scanned

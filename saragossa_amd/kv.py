@@ -123,6 +123,22 @@ class FullAttentionState:
         check(self._l.skv_attention_host(self._h, _p(qa), qa.size, window_start, _p(out)))
         return out
 
+    def prefill_rows(self, q, k, v) -> np.ndarray:
+        """cached_attention_prefill_rows (src/decoder/attention_ops.rs:976-1017): append the
+        rows of k/v and attend each new row causally over the cache. Host arrays."""
+        qa, ka, va = np.atleast_2d(_f32(q)), np.atleast_2d(_f32(k)), np.atleast_2d(_f32(v))
+        n = qa.shape[0]
+        if ka.shape != (n, self.kv_dim()) or va.shape != ka.shape or \
+                qa.shape[1] != self.q_heads() * self.head_dim():
+            from ._lib import DimensionError
+            raise DimensionError(f"attention batch cached shapes q={qa.shape}, k={ka.shape}, v={va.shape}")
+        out = np.empty_like(qa)
+        check(self._l.skv_prefill_chunk_host(self._h, _p(qa), _p(ka), _p(va), n, _p(out)))
+        return out
+
+    def encode_prefill_rows(self, stream, q_ptr, k_ptr, v_ptr, n_rows, out_ptr) -> None:
+        check(self._l.skv_prefill_chunk_device(self._h, stream, q_ptr, k_ptr, v_ptr, n_rows, out_ptr))
+
     def read_rows(self, first: int = 0, n: int | None = None):
         """Logical rows as bf16 bit patterns, ([n, kv_dim] uint16, same)."""
         n = self.len() - first if n is None else n

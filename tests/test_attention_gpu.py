@@ -190,3 +190,67 @@ def test_normal_inputs_config0(state):
     assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
     delta = np.abs(gpu - want)
     assert delta.max() <= 1e-4, delta.max()
+
+
+# ---- chunked prefill over the cache (multi-query, matrix cores) ----------------------------
+@pytest.mark.parametrize("dims,start,chunk,window", [
+    ((32, 8, 128), 0, 64, 0),        # first chunk from an empty cache
+    ((32, 8, 128), 300, 200, 0),     # later chunk, crosses page boundaries
+    ((16, 2, 256), 1000, 37, 0),     # head_dim 256, ragged chunk
+    ((16, 2, 256), 5, 3, 0),         # speculative-verify sized chunk (split over the context)
+    ((4, 2, 16), 0, 50, 0),
+    ((6, 1, 40), 17, 33, 0),         # head_dim padded to 64, GQA 6
+])
+def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk, window):
+    """One launch == the reference's per-row loop (append, then cached_attention_one)."""
+    q_heads, kv_heads, head_dim = dims
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(start * 7 + chunk)
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r")
+    kv = state.full_attention_bf16(start + chunk, q_heads, kv_heads, head_dim)
+    kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+    if start:
+        k0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+        v0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+        kv.seed(k0, v0, start)
+        cache.append_batch(k0, v0, lay)
+    q = rng.standard_normal((chunk, q_dim), dtype=np.float32)
+    k = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+    v = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+    got = kv.prefill_rows(q, k, v)
+    want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+    assert kv.len() == len(cache) == start + chunk
+    assert np.abs(got - want).max() <= 1e-4, np.abs(got - want).max()
+    gk, gv = kv.read_rows_f32()
+    assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
+
+
+@pytest.mark.parametrize("window,chunks", [(32, [40, 7, 64]), (20, [5, 30, 3])])
+def test_prefill_rows_on_ring_layer(state, window, chunks):
+    """A ring that holds exactly its window advances row by row; results equal the oracle's
+    sliding-window attention."""
+    q_heads, kv_heads, head_dim = 8, 2, 64
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(window)
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r")
+    kv = state.full_attention_bf16(sum(chunks), q_heads, kv_heads, head_dim, window=window)
+    for c in chunks:
+        q = rng.standard_normal((c, q_dim), dtype=np.float32)
+        k = rng.standard_normal((c, kv_dim), dtype=np.float32)
+        v = rng.standard_normal((c, kv_dim), dtype=np.float32)
+        got = kv.prefill_rows(q, k, v)
+        want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+        assert np.abs(got - want).max() <= 1e-4
+
+
+def test_prefill_rows_errors(state):
+    kv = state.full_attention_bf16(8, 4, 2, 16)
+    with pytest.raises(skv.DimensionError):
+        kv.prefill_rows(np.zeros((0, 64)), np.zeros((0, 32)), np.zeros((0, 32)))
+    with pytest.raises(skv.DimensionError):
+        kv.prefill_rows(np.zeros((2, 64)), np.zeros((3, 32)), np.zeros((2, 32)))
+    with pytest.raises(skv.DimensionError):
+        kv.prefill_rows(np.zeros((9, 64)), np.zeros((9, 32)), np.zeros((9, 32)))   # over capacity
+    assert kv.len() == 0
