@@ -24,6 +24,7 @@ __device__ __forceinline__ float xor_max(float v, int mask) {
 constexpr int DEC_MAX_SPLITS = 512;
 int decode_max_splits() { return DEC_MAX_SPLITS; }
 
+
 // ------------------------------------------------------------------------------------
 // Decode attention, split-K over the context, one workgroup per (split, kv head).
 //
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
 
-    // ---- all wavefronts publish (o, m, l); the workgroup reduces them column-parallel -------
+    // ---- all wavefronts publish (o, m, l); the workgroup reduces them, four columns per thread
     __syncthreads(); // the staged queries are no longer needed: the LDS is reused
     float *xo = reinterpret_cast<float *>(smem);        // [WAVES][rows][OSTRIDE]
     float *xm = xo + WAVES * rows * OSTRIDE;            // [WAVES][rows]
@@ -345,32 +346,49 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
         }
     }
     __syncthreads();
-    for (int idx = tid; idx < rows * P; idx += THREADS) {
-        const int row = idx / P;
-        const int col = idx - row * P;
+    constexpr int P4 = P / 4;
+    const bool vec_ok = (g.head_dim & 3) == 0;
+    for (int u = tid; u < rows * P4; u += THREADS) {
+        const int row = u / P4;
+        const int c4 = (u - row * P4) * 4;
+        float mw[WAVES];
         float mx = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, xm[w * rows + row]);
+        for (int w = 0; w < WAVES; ++w) {
+            mw[w] = xm[w * rows + row];
+            mx = fmaxf(mx, mw[w]);
+        }
         const float m_safe = mx == -INFINITY ? 0.0f : mx;
-        float acc = 0.0f, lsum = 0.0f;
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        float lsum = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; ++w) {
-            const float wgt = fast_exp2(xm[w * rows + row] - m_safe);
-            acc += wgt * xo[(w * rows + row) * OSTRIDE + col];
+            const float wgt = fast_exp2(mw[w] - m_safe);
+            acc += wgt * *reinterpret_cast<const float4_t *>(&xo[(w * rows + row) * OSTRIDE + c4]);
             lsum += wgt * xl[w * rows + row];
         }
-        if (col < g.head_dim) {
-            const int slot = tile * 16 + row;
-            if (a.splits == 1) {
-                a.out[((long)(slot / G) * g.q_heads + kvh * G + slot % G) * g.head_dim + col] = acc / lsum;
-            } else {
-                const long pidx = ((long)kvh * a.splits + split) * n_slots + slot;
-                a.part_o[pidx * g.head_dim + col] = acc;
-                if (col == 0) {
-                    a.part_m[pidx] = mx;
-                    a.part_l[pidx] = lsum;
-                }
+        if (c4 >= g.head_dim) continue;
+        const int slot = tile * 16 + row;
+        float *dst;
+        if (a.splits == 1) {
+            acc *= 1.0f / lsum;
+            dst = a.out + ((long)(slot / G) * g.q_heads + kvh * G + slot % G) * g.head_dim + c4;
+        } else {
+            const long pidx = ((long)kvh * a.splits + split) * n_slots + slot;
+            dst = a.part_o + pidx * g.head_dim + c4;
+            if (c4 == 0) {
+                a.part_m[pidx] = mx;
+                a.part_l[pidx] = lsum;
             }
+        }
+        if (vec_ok) {
+            // partials are read once by another kernel: keep them out of the caches
+            if (a.splits == 1) *reinterpret_cast<float4_t *>(dst) = acc;
+            else __builtin_nontemporal_store(acc, reinterpret_cast<float4_t *>(dst));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (c4 + i < g.head_dim) dst[i] = acc[i];
         }
     }
 }

@@ -257,7 +257,8 @@ void skv_ctx_destroy(skv_ctx *ctx) {
 
 int32_t skv_ctx_synchronize(skv_ctx *ctx) {
     if (!ctx) return fail(SKV_ERR_DEVICE, "ctx nul");
-    SKV_HIP(hipStreamSynchronize(ctx->stream));
+    SKV_HIP(hipSetDevice(ctx->device));
+    SKV_HIP(hipDeviceSynchronize());
     return SKV_OK;
 }
 
