@@ -1,0 +1,136 @@
+"""BASELINE.json configurations at their real shapes (layer counts reduced where a layer is
+a repeat of another), against the CPU oracle: cache contents bit-exact, attention within 1e-4
+(bound held to: 1e-2), plus size-independent properties at full size."""
+import numpy as np
+import pytest
+
+import oracle
+import saragossa_amd as skv
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _seed_device(kv, rows, kv_dim, gen):
+    k = torch.randn(rows, kv_dim, device="cuda", dtype=torch.float32, generator=gen)
+    v = torch.randn(rows, kv_dim, device="cuda", dtype=torch.float32, generator=gen)
+    kv.encode_append_batch(_stream(), k.data_ptr(), v.data_ptr(), rows)
+    torch.cuda.synchronize()
+    return k.cpu().numpy(), v.cpu().numpy()
+
+
+def test_config2_hybrid_32k_decode_steps(state):
+    """configs[2]: full-attention layers 16/2/256 at 32768 cached rows (2 of the 10 identical
+    layers), random block tables, decode steps with fresh q, k, v; the 30 recurrent states
+    (96 KiB conv + 2 MiB ssm each) are snapshotted once and restored byte-identically."""
+    qh, kvh, hd, ctx, steps, n_layers = 16, 2, 256, 32768, 6, 2
+    kv_dim, q_dim = kvh * hd, qh * hd
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    rng = np.random.default_rng(2)
+    lay = oracle.layout(qh, kvh, hd)
+    layers, caches = [], []
+    for _ in range(n_layers):
+        kv = state.full_attention_bf16(ctx + steps, qh, kvh, hd)
+        kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+        k, v = _seed_device(kv, ctx, kv_dim, gen)
+        c = oracle.LayerKvCache("bf16r")
+        c.append_batch(k, v, lay)
+        layers.append(kv)
+        caches.append(c)
+    qs = torch.randn(steps, n_layers, q_dim, device="cuda", generator=gen)
+    ks = torch.randn(steps, n_layers, kv_dim, device="cuda", generator=gen)
+    vs = torch.randn(steps, n_layers, kv_dim, device="cuda", generator=gen)
+    out = torch.empty(steps, n_layers, q_dim, device="cuda")
+    for t in range(steps):
+        for li, kv in enumerate(layers):
+            kv.encode_decode_step(_stream(), ks[t, li].data_ptr(), 0, vs[t, li].data_ptr(), 0,
+                                  qs[t, li].data_ptr(), out[t, li].data_ptr())
+    got = out.cpu().numpy()
+    qn, kn, vn = qs.cpu().numpy(), ks.cpu().numpy(), vs.cpu().numpy()
+    worst = 0.0
+    for t in range(steps):
+        for li in range(n_layers):
+            want = oracle.decode_step(caches[li], kn[t, li], vn[t, li], qn[t, li], lay)
+            worst = max(worst, float(np.abs(got[t, li] - want).max()))
+    assert worst <= 1e-4, worst
+    for kv, c in zip(layers, caches):
+        gk, gv = kv.read_rows_f32(ctx - 40, 40 + steps)
+        assert np.array_equal(gk, c.keys()[ctx - 40:]) and np.array_equal(gv, c.values()[ctx - 40:])
+    # recurrent state: snapshot once, clobber, restore
+    sizes = [3 * 8192 * 4, 32 * 128 * 128 * 4] * 30
+    bufs = [torch.randn(s // 4, device="cuda", generator=gen) for s in sizes]
+    keep = [b.clone() for b in bufs]
+    snap = skv.state_snapshot(state, [b.data_ptr() for b in bufs], sizes, stream=_stream())
+    assert snap.estimated_bytes() == sum(sizes)
+    for b in bufs:
+        b.add_(1.0)
+    skv.state_restore(state, snap, [b.data_ptr() for b in bufs], sizes, stream=_stream())
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(bufs, keep))
+
+
+def test_config4_sliding_window_model_batch1_and_batch4(state):
+    """configs[4]: 16/8/256, local layers keep a 1024-token ring, global layers the full paged
+    cache at 65536 rows, local:global 5:1 (one group of six layers); decode steps at batch 1
+    and at batch 4 with independent sequences that own their tables."""
+    qh, kvh, hd, ctx, window = 16, 8, 256, 65536, 1024
+    kv_dim, q_dim = kvh * hd, qh * hd
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    rng = np.random.default_rng(4)
+
+    def build_sequence(steps):
+        layers, caches, lays = [], [], []
+        for li in range(6):
+            is_global = (li + 1) % 6 == 0          # src/decoder.rs:890-898
+            w = 0 if is_global else window
+            kv = state.full_attention_bf16(ctx + steps, qh, kvh, hd, window=w)
+            kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+            lay = oracle.layout(qh, kvh, hd, sliding_window=w)
+            c = oracle.LayerKvCache("bf16r")
+            if is_global:
+                k, v = _seed_device(kv, ctx, kv_dim, gen)
+                c.append_batch(k, v, lay)
+            else:
+                # a local layer only ever attends its last `window` rows, so it starts with its
+                # ring exactly full (position 1024) and wraps from the first decode step on
+                k, v = _seed_device(kv, window, kv_dim, gen)
+                c.append_batch(k, v, lay)
+            layers.append(kv)
+            caches.append(c)
+            lays.append(lay)
+        return layers, caches, lays
+
+    def run(seqs, steps):
+        worst = 0.0
+        for t in range(steps):
+            for layers, caches, lays in seqs:
+                for kv, c, lay in zip(layers, caches, lays):
+                    q = torch.randn(q_dim, device="cuda", generator=gen)
+                    k = torch.randn(kv_dim, device="cuda", generator=gen)
+                    v = torch.randn(kv_dim, device="cuda", generator=gen)
+                    o = torch.empty(q_dim, device="cuda")
+                    kv.encode_decode_step(_stream(), k.data_ptr(), 0, v.data_ptr(), 0, q.data_ptr(),
+                                          o.data_ptr())
+                    want = oracle.decode_step(c, k.cpu().numpy(), v.cpu().numpy(), q.cpu().numpy(), lay)
+                    worst = max(worst, float(np.abs(o.cpu().numpy() - want).max()))
+        return worst
+
+    one = [build_sequence(4)]
+    assert run(one, 4) <= 1e-4
+    # ring layers hold exactly their window after wrapping; global layer keeps everything
+    layers, caches, _ = one[0]
+    assert layers[0].pages() == window // 16 and layers[5].pages() == (ctx + 4 + 15) // 16
+    gk, _ = layers[0].read_rows_f32(layers[0].len() - window, window)
+    assert np.array_equal(gk, caches[0].keys()[-window:])
+    for kv in layers:
+        kv.close()
+    four = [build_sequence(3) for _ in range(4)]
+    assert run(four, 3) <= 1e-4
+    # sequences are independent: same layer index, different contents
+    a, _ = four[0][0][5].read_rows(ctx, 3)
+    b, _ = four[1][0][5].read_rows(ctx, 3)
+    assert not np.array_equal(a, b)
