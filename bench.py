@@ -29,7 +29,18 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 
-CFG = dict(layers=10, q_heads=16, kv_heads=2, head_dim=256, context=32768)
+# BASELINE.json configs that are decode workloads. Each entry: groups of identical layers
+# (count, q_heads, kv_heads, head_dim, cached rows, sliding window). The default, and the
+# configuration the metric is quoted on, is configs[2].
+WORKLOADS = {
+    1: dict(name="configs[1]: 36 layers q32/kv8/hd128 (Qwen3-4B KV shapes), %d cached rows",
+            groups=[(36, 32, 8, 128, 2048, 0)]),
+    2: dict(name="configs[2]: 10 full-attention layers q16/kv2/hd256, %d cached rows",
+            groups=[(10, 16, 2, 256, 32768, 0)]),
+    4: dict(name="configs[4]: 8 global layers q16/kv8/hd256 at %d rows + 40 local layers with a "
+                 "1024-row ring",
+            groups=[(8, 16, 8, 256, 65536, 0), (40, 16, 8, 256, 65536, 1024)]),
+}
 
 
 def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> int:
@@ -119,7 +130,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--context", type=int, default=CFG["context"])
+    ap.add_argument("--config", type=int, default=2, choices=sorted(WORKLOADS))
+    ap.add_argument("--context", type=int, default=0, help="override the cached rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-restore", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -139,30 +151,38 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    layers_n, qh, kvh, hd = CFG["layers"], CFG["q_heads"], CFG["kv_heads"], CFG["head_dim"]
+    wl = WORKLOADS[args.config]
+    if len(wl["groups"]) > 1:
+        args.no_cpu_baseline = True   # the CPU sample is scaled by identical layers only
+    groups = [(n, qh_, kvh_, hd_, args.context or ctx_, w_) for n, qh_, kvh_, hd_, ctx_, w_ in wl["groups"]]
+    qh, kvh, hd = groups[0][1:4]     # all groups of a workload share the head shape
     kv_dim, q_dim = kvh * hd, qh * hd
-    ctx_rows = args.context
+    ctx_rows = groups[0][4]
+    layers_n = sum(g[0] for g in groups)
     total_steps = args.warmup + args.steps
-    capacity = ctx_rows + 2 * total_steps + 8
 
     gen = torch.Generator(device=dev)
-    gen.manual_seed(2)
-    rng = np.random.default_rng(2)
+    gen.manual_seed(args.config)
+    rng = np.random.default_rng(args.config)
     state = skv.DecodeResidentState(0)
     stream = torch.cuda.current_stream().cuda_stream
     layers = []
-    host_kv = []  # first layer's f32 rows, kept for the CPU baseline
-    for li in range(layers_n):
-        kv = state.full_attention_bf16(capacity, qh, kvh, hd)
-        kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
-        k = torch.randn(ctx_rows, kv_dim, device=dev, dtype=torch.float32, generator=gen)
-        v = torch.randn(ctx_rows, kv_dim, device=dev, dtype=torch.float32, generator=gen)
-        kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), ctx_rows)
-        torch.cuda.synchronize()
-        if li == 0 and not args.no_cpu_baseline:
-            host_kv = [k.cpu().numpy(), v.cpu().numpy()]
-        del k, v
-        layers.append(kv)
+    layer_rows = []   # rows each layer attends per step (for the byte count)
+    host_kv = []      # first layer's f32 rows, kept for the CPU baseline
+    for n, _, _, _, rows, window in groups:
+        for _ in range(n):
+            kv = state.full_attention_bf16(rows + 2 * total_steps + 8, qh, kvh, hd, window=window)
+            kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+            fill = min(rows, window) if window else rows   # a ring only keeps its window
+            k = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+            v = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+            kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), fill)
+            torch.cuda.synchronize()
+            if not layers and not args.no_cpu_baseline:
+                host_kv = [k.cpu().numpy(), v.cpu().numpy()]
+            del k, v
+            layers.append(kv)
+            layer_rows.append(fill)
 
     n_pass = 2 * total_steps  # timed pass + per-kernel pass
     q_all = torch.randn(n_pass, layers_n, q_dim, device=dev, dtype=torch.float32, generator=gen)
@@ -198,8 +218,9 @@ def main() -> int:
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     us_per_token = ms_per_step * 1e3
-    rows_mid = ctx_rows + args.warmup + args.steps // 2
-    step_bytes = layers_n * algorithmic_bytes(rows_mid, kv_dim, q_dim, with_append=True)
+    mid = args.warmup + args.steps // 2
+    step_bytes = sum(algorithmic_bytes(min(r + mid, w) if w else r + mid, kv_dim, q_dim, True)
+                     for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
 
     # ---- per-kernel pass on the launch stream: the ten appends of a token first, then HIP
     # events around the ten attention launches (one per layer) so that the cost of recording
@@ -213,15 +234,20 @@ def main() -> int:
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
         for li, kv in enumerate(layers):
-            kv.encode_attention_decode(stream, qp[li], out_arr[li])
+            ws = max(kv.len() - kv.window(), 0) if kv.window() else 0
+            kv.encode_attention_decode_windowed(stream, qp[li], out_arr[li], ws)
         e1.record()
         evs.append((e0, e1))
     torch.cuda.synchronize()
     kern_ms = sorted(e0.elapsed_time(e1) / layers_n for e0, e1 in evs)
     kern_avg_us = sum(kern_ms) / len(kern_ms) * 1e3
     kern_med_us = kern_ms[len(kern_ms) // 2] * 1e3
-    rows_k = ctx_rows + total_steps + args.steps // 2
-    launch_bytes = algorithmic_bytes(rows_k, kv_dim, q_dim, with_append=False)
+    # the dominant launch is a layer of the first group; with mixed groups the event pairs span
+    # all layers, so bytes are summed over the layers and divided by the same time
+    late = total_steps + args.steps // 2
+    all_bytes = sum(algorithmic_bytes(min(r + late, w) if w else r + late, kv_dim, q_dim, False)
+                    for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
+    launch_bytes = all_bytes // layers_n
     achieved = launch_bytes / (kern_avg_us * 1e-6) / 1e9
     cpu_inputs = None
     if not args.no_cpu_baseline:
@@ -231,10 +257,11 @@ def main() -> int:
     del layers, q_all, k_all, v_all
     torch.cuda.empty_cache()
 
-    restore = None if args.no_restore else bench_restore(skv, torch, np, state, stream)
+    restore = None if (args.no_restore or args.config != 2) else bench_restore(skv, torch, np, state, stream)
 
     result = {
-        "metric": "KV-path decode us/token @32k ctx (append + paged GQA SDPA, 10 KV layers)",
+        "metric": "KV-path decode us/token @32k ctx (append + paged GQA SDPA, 10 KV layers)"
+                  if args.config == 2 else "KV-path decode us/token (append + paged GQA SDPA)",
         "value": round(us_per_token, 2),
         "unit": "us/token",
         "n_gpus": 1,
@@ -246,14 +273,14 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "configs[2]: 10 full-attention layers q16/kv2/hd256, bf16 KV in "
-                               "16-token pages, %d cached rows, batch 1, 1 token per step"
-                               % ctx_rows,
+        "config": {"workload": (wl["name"] % ctx_rows) + ", bf16 KV in 16-token pages, batch 1, "
+                               "1 token per step",
                    "context": ctx_rows, "layers": layers_n, "page_rows": 16},
         "tok_per_s": round(1e6 / us_per_token, 1),
         "hbm_gbps": round(step_bytes / (us_per_token * 1e-6) / 1e9, 1),
         "hbm_frac": round(step_bytes / (us_per_token * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel<256,8> + decode_merge_kernel (one attention launch)",
+        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
+                               "average over the layers)" % (128 if hd <= 128 else 256),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "bytes_per_launch": launch_bytes,

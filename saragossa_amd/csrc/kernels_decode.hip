@@ -400,8 +400,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
 // and the two sums are then reduced across the split lanes through LDS.
 // Stands in for attention_decode_2pass_2 (src/decode_resident/kernels.rs:801-917).
 // ------------------------------------------------------------------------------------
-constexpr int MERGE_PER_LANE = DEC_MAX_SPLITS / 16;
+constexpr int MERGE_PER_LANE_MAX = DEC_MAX_SPLITS / 16;
 
+// MERGE_PER_LANE: splits each of the 16 split lanes covers, the smallest power of two that fits
+template <int MERGE_PER_LANE>
 __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
     const Geom g = a.g;
     const int n_slots = a.n_queries * g.gqa;
@@ -495,7 +497,13 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     }
     if (e != hipSuccess || a.splits == 1) return e;
     dim3 mgrid((unsigned)(a.g.kv_heads * a.n_queries * a.g.gqa), (unsigned)((a.g.head_dim + 15) / 16));
-    hipLaunchKernelGGL(decode_merge_kernel, mgrid, dim3(256), 0, s, a);
+    const int per_lane = (a.splits + 15) / 16;
+    if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_kernel<1>, mgrid, dim3(256), 0, s, a);
+    else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_kernel<2>, mgrid, dim3(256), 0, s, a);
+    else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_kernel<4>, mgrid, dim3(256), 0, s, a);
+    else if (per_lane <= 8) hipLaunchKernelGGL(decode_merge_kernel<8>, mgrid, dim3(256), 0, s, a);
+    else if (per_lane <= 16) hipLaunchKernelGGL(decode_merge_kernel<16>, mgrid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(decode_merge_kernel<MERGE_PER_LANE_MAX>, mgrid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -1,0 +1,53 @@
+"""BASELINE configs[1]: random-init Qwen3-4B-shaped decoder, chunked prefill over the cache,
+then greedy decode; token ids with the HIP KV path must equal the ids with the CPU oracle's
+KV path, and the caches must hold the same bf16 rows. The default run uses 4 of the 36 layers
+and a 256-token prompt so that the oracle's per-row CPU prefill stays within the suite's time
+budget; SKV_FULL_CONFIG1=1 runs the full 36 layers, 2048-token prompt and 256 steps (several
+minutes of CPU attention)."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+from config1_model import Config, HipKv, OracleKv, Weights, greedy  # noqa: E402
+
+FULL = os.environ.get("SKV_FULL_CONFIG1") == "1"
+
+
+@pytest.mark.timeout(3000 if FULL else 300)
+def test_config1_greedy_ids_match_oracle(state):
+    cfg = Config() if FULL else Config(layers=4)
+    n_prompt, n_new, chunk = (2048, 256, 512) if FULL else (256, 48, 96)
+    w = Weights(cfg, seed=1)
+    prompt = [int(t) for t in np.random.default_rng(1).integers(0, cfg.vocab, size=n_prompt)]
+    cap = n_prompt + n_new
+    with torch.no_grad():
+        hip = HipKv(cfg, cap, state)
+        ids_hip, margins, logits_hip = greedy(cfg, w, hip, prompt, n_new, chunk)
+        ora = OracleKv(cfg)
+        ids_ora, _, logits_ora = greedy(cfg, w, ora, prompt, n_new, chunk)
+    print(f"config1 {'full' if FULL else 'reduced'}: min top-1/top-2 margin {min(margins):.3e}, "
+          f"max |logit diff| {max(float(np.abs(a - b).max()) for a, b in zip(logits_hip, logits_ora)):.3e}")
+    first_diff = next((i for i, (a, b) in enumerate(zip(ids_hip, ids_ora)) if a != b), None)
+    if first_diff is not None:
+        print(f"first differing step {first_diff}: margin there {margins[first_diff]:.3e}")
+    assert ids_hip == ids_ora
+    assert len(set(ids_hip)) > 1          # not a degenerate constant continuation
+    # Cache contents after the run. Layer 0's K/V depend on the embeddings only, so both arms
+    # append the same f32 rows and the caches must agree bit for bit. Deeper layers receive
+    # hidden states that already carry the arms' last-bit attention differences; bf16 rounding
+    # of K/V amplifies those (a 1e-6 change tips a rounding now and then, the tipped element
+    # moves the next layer's scores by 1e-4), so there the appended inputs themselves differ and
+    # only closeness is checked.
+    for li in sorted({0, cfg.layers // 2, cfg.layers - 1}):
+        gk, gv = hip.contents(li)
+        ok, ov = ora.contents(li)
+        assert gk.shape == ok.shape == (cap, cfg.kv_heads * cfg.head_dim)
+        if li == 0:
+            assert np.array_equal(gk, ok) and np.array_equal(gv, ov)
+        else:
+            for g, o in ((gk, ok), (gv, ov)):
+                assert np.abs(g - o).max() <= 0.1 and np.abs(g - o).mean() <= 1e-3
