@@ -276,6 +276,14 @@ int32_t skv_hot_remember(skv_hot *hot, skv_stream stream, const uint8_t session[
                          const uint8_t hash[32], size_t tokens, skv_layer *const *layers,
                          size_t n_layers, const void *const *state_ptrs, const size_t *state_bytes,
                          size_t n_states, int32_t *cached);
+/* remember_prefix_block for n_blocks consecutive boundaries (first_tokens, first_tokens +
+ * block_tokens, ...) keyed by hashes[i] (n_blocks x 32 bytes): the same evictions and
+ * insertions in the same order as separate calls, with the page copies queued together. What
+ * the block-boundary loop of prefill_prompt_state (src/serve/state.rs:595-602) does after a
+ * chunk that spans several blocks. No recurrent state. *n_cached counts the blocks kept. */
+int32_t skv_hot_remember_range(skv_hot *hot, skv_stream stream, const uint8_t session[32],
+                               const uint8_t *hashes, size_t first_tokens, size_t n_blocks,
+                               skv_layer *const *layers, size_t n_layers, size_t *n_cached);
 /* The hit branch of prefill_prompt_state (src/serve/state.rs:574-584): longest cached
  * chain for `tokens` under `root`, its pages gathered into rows [0, *reused_tokens) of the
  * layers, the last block's recurrent state copied to state_ptrs, each layer's len set to

@@ -10,10 +10,11 @@ from ._lib import (KvError, DimensionError, ConfigError, DeviceError, lib, lib_p
                    DTYPE_BF16, DTYPE_F32, PAGE_ROWS)
 from .kv import DecodeResidentState, FullAttentionState
 from . import flags
+from .serve import LoadedModelKv
 from .prefix import (BlockHash, BlockAwarePrefixCache, PrefixBlockHit, HotCache, Snapshot,
                      snapshot_blocks, restore_blocks, state_snapshot, state_restore)
 
 __all__ = ["KvError", "DimensionError", "ConfigError", "DeviceError", "lib", "lib_path",
            "DecodeResidentState", "FullAttentionState", "flags", "DTYPE_BF16", "DTYPE_F32",
            "PAGE_ROWS", "BlockHash", "BlockAwarePrefixCache", "PrefixBlockHit", "HotCache",
-           "Snapshot", "snapshot_blocks", "restore_blocks", "state_snapshot", "state_restore"]
+           "LoadedModelKv", "Snapshot", "snapshot_blocks", "restore_blocks", "state_snapshot", "state_restore"]

@@ -116,6 +116,7 @@ SIGNATURES = {
     "skv_hot_destroy": (None, [_vp]),
     "skv_hot_remember": (_i32, [_vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz,
                                 C.POINTER(_i32)]),
+    "skv_hot_remember_range": (_i32, [_vp, _vp, _vp, _vp, _sz, _sz, _vp, _sz, C.POINTER(_sz)]),
     "skv_hot_match_restore": (_i32, [_vp, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz,
                                      C.POINTER(_sz), _vp]),
     "skv_hot_evict_lru": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_sz)]),

@@ -539,6 +539,95 @@ int32_t skv_hot_remember(skv_hot *h, skv_stream stream, const uint8_t session[32
     return SKV_OK;
 }
 
+// remember_prefix_block for `n_blocks` consecutive boundaries in one call: block i covers
+// rows [first_tokens - block_tokens + i*block_tokens, first_tokens + i*block_tokens) and is
+// keyed by hashes[i]. Same evictions and insertions, in the same order, as n_blocks separate
+// calls; the page copies of all blocks are queued together. For caches without recurrent
+// state (a state exists only at the boundary the decoder is at).
+int32_t skv_hot_remember_range(skv_hot *h, skv_stream stream, const uint8_t session[32],
+                               const uint8_t *hashes, size_t first_tokens, size_t n_blocks,
+                               skv_layer *const *layers, size_t n_layers, size_t *n_cached) {
+    if (!h || !session || (n_blocks && !hashes)) return fail(SKV_ERR_DEVICE, "hot_remember_range: pointeur nul");
+    if (n_cached) *n_cached = 0;
+    int32_t rc = check_layers(h->ctx, layers, n_layers);
+    if (rc) return rc;
+    if (!h->layout.matches(layers, n_layers))
+        return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: les couches n'ont pas la forme du pool");
+    const size_t bt = h->index->block_tokens();
+    if (n_blocks == 0) return SKV_OK;
+    if (first_tokens < bt || first_tokens % bt != 0)
+        return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: tokens=" + std::to_string(first_tokens) +
+                                           " n'est pas une frontière de bloc");
+    const size_t last_tokens = first_tokens + (n_blocks - 1) * bt;
+    for (size_t l = 0; l < n_layers; ++l) {
+        if (layers[l]->len < last_tokens)
+            return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: couche plus courte que la frontière");
+        if (layers[l]->g.ring_rows > 0 && first_tokens - bt < layers[l]->floor_pos)
+            return fail(SKV_ERR_DIMENSION, "prefix-cache GPU: bloc déjà évincé de l'anneau");
+    }
+    if (h->index->capacity() == 0) return SKV_OK;
+    SKV_HIP(hipSetDevice(h->ctx->device));
+    std::vector<int32_t> pages, slots;
+    std::vector<char> pending(h->pool_slots, 0); // slots written by copies not yet queued
+    auto flush = [&]() -> int32_t {
+        if (pages.empty()) return SKV_OK;
+        int32_t r = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(),
+                               pages.size(), nullptr, true, as_stream(stream));
+        for (int32_t sl : slots) pending[sl] = 0;
+        pages.clear();
+        slots.clear();
+        return r;
+    };
+    size_t cached = 0;
+    for (size_t b = 0; b < n_blocks; ++b) {
+        const size_t tokens = first_tokens + b * bt;
+        bool skipped = false;
+        while (h->free_slots.size() < h->pages_per_block) {
+            uint64_t id = 0;
+            if (!h->index->evict_lru(&id, nullptr)) {
+                ++h->skipped;
+                skipped = true;
+                break;
+            }
+            hot_release(h, id);
+            ++h->evictions;
+        }
+        if (skipped) continue;
+        HotEntry e;
+        bool reuse = false;
+        for (size_t i = 0; i < h->pages_per_block; ++i) {
+            const int32_t sl = h->free_slots.back();
+            h->free_slots.pop_back();
+            e.slots.push_back(sl);
+            reuse = reuse || pending[sl];
+        }
+        if (reuse) { // a slot freed by an eviction inside this call: its old copy goes first
+            rc = flush();
+            if (rc) return rc;
+        }
+        for (size_t i = 0; i < h->pages_per_block; ++i) {
+            pages.push_back((int32_t)((tokens - bt) / 16 + i));
+            slots.push_back(e.slots[i]);
+            pending[e.slots[i]] = 1;
+        }
+        e.bytes = h->pages_per_block * h->layout.slot_bytes;
+        const uint64_t id = h->next_id++;
+        const size_t nbytes = e.bytes;
+        h->entries.emplace(id, std::move(e));
+        std::vector<uint64_t> dropped;
+        h->index->insert(session, hashes + 32 * b, tokens, id, nbytes, &dropped);
+        for (uint64_t d : dropped) {
+            if (d != id) ++h->evictions;
+            hot_release(h, d);
+        }
+        if (h->entries.count(id)) ++cached;
+    }
+    rc = flush();
+    if (rc) return rc;
+    if (n_cached) *n_cached = cached;
+    return SKV_OK;
+}
+
 // The hit branch of prefill_prompt_state (src/serve/state.rs:574-584): longest chain of
 // cached blocks for `tokens`, every matched block's pages copied into the layers' rows
 // [0, reused), the recurrent state of the last matched block copied out, len = reused.

@@ -258,6 +258,17 @@ class HotCache:
                                        sa if n else None, n, C.byref(cached)))
         return bool(cached.value)
 
+    def remember_prefix_blocks(self, session: bytes, hashes, first_tokens: int, layers,
+                               stream=None) -> int:
+        """remember_prefix_block for consecutive boundaries; returns how many were kept."""
+        blob = b"".join(hashes)
+        buf = (C.c_uint8 * len(blob)).from_buffer_copy(blob) if blob else None
+        kept = C.c_size_t()
+        check(self._l.skv_hot_remember_range(self._h, stream, _in32(session), buf, first_tokens,
+                                             len(hashes), _layer_array(layers), len(layers),
+                                             C.byref(kept)))
+        return kept.value
+
     def match_restore(self, root: bytes, tokens, layers, state_ptrs=(), state_sizes=(),
                       stream=None):
         """Returns (reused_tokens, hash of the last reused block or None)."""

@@ -136,12 +136,15 @@ class SimDecoder(pc.PromptDecoder):
     def extend(self, state, tokens): state.n += len(tokens)
 
 
-@pytest.mark.parametrize("dims,n_layers,bt,prefix,pool_frac", [
-    ((32, 8, 128), 4, 16, 256, 0.6),     # BASELINE config 3 shapes, scaled down
-    ((16, 2, 256), 2, 32, 128, 0.5),     # two pages per hash block
+@pytest.mark.parametrize("dims,n_layers,bt,prefix,pool_frac,chunk_blocks", [
+    ((32, 8, 128), 4, 16, 256, 0.6, 1),  # BASELINE config 3 shapes, scaled down
+    ((16, 2, 256), 2, 32, 128, 0.5, 1),  # two pages per hash block
+    ((32, 8, 128), 3, 16, 256, 0.6, 8),  # several blocks prefilled and remembered per call
+    ((32, 8, 128), 2, 16, 128, 0.15, 5), # a pool so small that blocks of one call evict each other
 ])
 def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims, n_layers, bt,
-                                                                     prefix, pool_frac):
+                                                                     prefix, pool_frac,
+                                                                     chunk_blocks):
     kv_dim = dims[1] * dims[2]
     rng = np.random.default_rng(33)
     n_sessions, vocab = 6, 151936
@@ -162,21 +165,16 @@ def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims
     over = lambda extra: len(ocache.entries) + extra > pool_blocks
     odec = SimDecoder()
 
+    model = skv.LoadedModelKv(hot, enabled=True)
+
     def run_turn(session_key, tokens):
         layers = make_layers(state, n_layers, cap, dims, seed=len(tokens))
-        root = BlockHash.for_session(session_key)
-        reused, h = hot.match_restore(root, tokens, layers, stream=_stream())
+        reused = model.prefill_prompt_state(
+            tokens, session_key, layers,
+            lambda first, last: fill(layers, first, last, tokens, kv_dim), stream=_stream(),
+            blocks_per_chunk=chunk_blocks)
         _, want_reused = pc.prefill_prompt_state(ocache, odec, tokens, session_key, over)
         assert reused == want_reused
-        h = h or root
-        consumed = reused
-        while consumed + bt <= len(tokens) // bt * bt:
-            fill(layers, consumed, consumed + bt, tokens, kv_dim)
-            h = BlockHash.chain(h, tokens[consumed:consumed + bt])
-            consumed += bt
-            hot.remember_prefix_block(root, h, consumed, layers, stream=_stream())
-        if consumed < len(tokens):
-            fill(layers, consumed, len(tokens), tokens, kv_dim)
         torch.cuda.synchronize()
         check_contents(layers, len(tokens), tokens, kv_dim)
         assert [(e["hash"], e["tokens"]) for e in hot.entries] == \
@@ -190,10 +188,19 @@ def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims
         total_reused += run_turn(None, shared + hist[s])
     for s in range(n_sessions):                 # second turn: everything so far + the new turn
         total_reused += run_turn(None, shared + hist[s] + turns[s])
-    assert total_reused > 0 and hot.evictions() > 0
+    assert hot.evictions() > 0 and (total_reused > 0 or pool_frac < 0.3)
     assert len(hot) <= pool_blocks and hot.free_blocks() == pool_blocks - len(hot)
     # sessions are isolated by their root
     assert run_turn("agent-a", shared + hist[0]) == 0
+    # the kill-switch path prefills everything and touches no cache state
+    before = [(e["hash"], e["tokens"]) for e in hot.entries]
+    off_layers = make_layers(state, n_layers, cap, dims, seed=5)
+    off_tokens = shared + hist[1]
+    assert skv.LoadedModelKv(hot, enabled=False).prefill_prompt_state(
+        off_tokens, None, off_layers,
+        lambda first, last: fill(off_layers, first, last, off_tokens, kv_dim)) == 0
+    check_contents(off_layers, len(off_tokens), off_tokens, kv_dim)
+    assert [(e["hash"], e["tokens"]) for e in hot.entries] == before
     # drain: evict_lru_block returns the bytes of each victim, then None
     n = len(hot)
     got = [hot.evict_lru_block() for _ in range(n)]
