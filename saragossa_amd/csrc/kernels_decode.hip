@@ -7,6 +7,7 @@ namespace skv {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) short short4_t;
 typedef __attribute__((ext_vector_type(4))) float float4_t;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 
 __device__ __forceinline__ uint16_t bf16_bits(float v) {
     uint32_t b = __float_as_uint(v);
@@ -56,17 +57,17 @@ template <int KK>
 __device__ __forceinline__ void load_k(uint4 (&k)[KK], const DecodeArgs &a, int page, int kvh,
                                        int lane) {
     const long tile = (long)page * a.g.page_elems + (long)kvh * a.g.tile_elems;
-    const uint4 *kp = reinterpret_cast<const uint4 *>(a.k_pool + tile) + lane;
+    const u32x4_t *kp = reinterpret_cast<const u32x4_t *>(a.k_pool + tile) + lane;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) k[kk] = kp[kk * 64];
+    for (int kk = 0; kk < KK; ++kk) k[kk] = __builtin_bit_cast(uint4, __builtin_nontemporal_load(kp + kk * 64));
 }
 template <int KK>
 __device__ __forceinline__ void load_v(uint4 (&v)[KK], const DecodeArgs &a, int page, int kvh,
                                        int lane) {
     const long tile = (long)page * a.g.page_elems + (long)kvh * a.g.tile_elems;
-    const uint4 *vp = reinterpret_cast<const uint4 *>(a.v_pool + tile) + lane;
+    const u32x4_t *vp = reinterpret_cast<const u32x4_t *>(a.v_pool + tile) + lane;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) v[kk] = vp[kk * 64];
+    for (int kk = 0; kk < KK; ++kk) v[kk] = __builtin_bit_cast(uint4, __builtin_nontemporal_load(vp + kk * 64));
 }
 
 template <int P, int WAVES>
