@@ -254,3 +254,77 @@ def test_prefill_rows_errors(state):
     with pytest.raises(skv.DimensionError):
         kv.prefill_rows(np.zeros((9, 64)), np.zeros((9, 32)), np.zeros((9, 32)))   # over capacity
     assert kv.len() == 0
+
+
+# ---- kill-switches -----------------------------------------------------------------------
+@pytest.fixture
+def env_flags():
+    saved = {}
+
+    def set_env(**kv):
+        for k, v in kv.items():
+            saved.setdefault(k, os.environ.get(k))
+            os.environ[k] = v
+        skv.flags.reload()
+
+    yield set_env
+    for k, v in saved.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
+    skv.flags.reload()
+
+
+@pytest.mark.parametrize("n,dims", [(1, (16, 2, 256)), (257, (16, 2, 256)), (4096, (16, 2, 256)),
+                                    (700, (4, 2, 16)), (300, (2, 1, 40))])
+def test_flash_sdpa_off_uses_plain_kernel(state, env_flags, n, dims):
+    """RETI_RUST_FLASH_SDPA=0 (src/decode_resident/utils.rs:182-185) selects the plain
+    three-phase kernel; its sequential sums track the CPU path more closely still."""
+    env_flags(RETI_RUST_FLASH_SDPA="0")
+    assert not skv.flags.flash_sdpa_enabled()
+    gpu = run_attention_case(state, n, *dims)
+    env_flags(RETI_RUST_FLASH_SDPA="1")
+    again = run_attention_case(state, n, *dims)
+    assert np.abs(gpu - again).max() <= 2e-5      # the two device kernels agree with each other
+
+
+def test_plain_kernel_handles_head_dim_512_and_windows(state, env_flags):
+    """head_dim above 256 is served by the plain kernel whatever the flag says; the windowed
+    entry masks the rows before window_start there too (the reference's naive kernel is its
+    windowed path, src/decode_resident/attention.rs:780-786)."""
+    q_heads, kv_heads, head_dim, n = 4, 2, 512, 90
+    kv_dim = kv_heads * head_dim
+    rng = np.random.default_rng(512)
+    keys = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    values = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    q = rng.standard_normal(q_heads * head_dim, dtype=np.float32)
+    kv = state.full_attention_bf16(n, q_heads, kv_heads, head_dim)
+    kv.seed(keys, values, n)
+    for ws in (0, 33):
+        got = kv.attention_decode_windowed(q, ws)
+        want = cpu_attention(q, keys[ws:], values[ws:], q_heads, kv_heads, head_dim)
+        assert np.abs(got - want).max() <= 1e-5
+    gk, _ = kv.read_rows_f32()
+    assert np.array_equal(gk, oracle.bf16_round(keys))
+
+
+def test_sdpa_2pass_off_and_min_len(state, env_flags):
+    """RETI_RUST_SDPA_2PASS=0 keeps one split; RETI_RUST_SDPA_2PASS_MIN_LEN moves the
+    switch-over (src/decode_resident/utils.rs:260-278). Results are split-independent to
+    fp32 rounding (the invariant that pins the merge)."""
+    base = run_attention_case(state, 3000, 32, 8, 128)
+    env_flags(RETI_RUST_SDPA_2PASS="0")
+    single = run_attention_case(state, 3000, 32, 8, 128)
+    env_flags(RETI_RUST_SDPA_2PASS="1", RETI_RUST_SDPA_2PASS_MIN_LEN="100000")
+    assert skv.flags.sdpa_2pass_min_len() == 100000
+    below = run_attention_case(state, 3000, 32, 8, 128)
+    assert np.abs(base - single).max() <= 2e-6 and np.array_equal(single, below)
+    for splits_env in ("64", "1024"):
+        os.environ["SKV_DECODE_WGS"] = splits_env
+        env_flags(RETI_RUST_SDPA_2PASS_MIN_LEN="128")
+        try:
+            other = run_attention_case(state, 3000, 32, 8, 128)
+        finally:
+            os.environ.pop("SKV_DECODE_WGS", None)
+        assert np.abs(base - other).max() <= 2e-6
