@@ -70,7 +70,9 @@ __device__ __forceinline__ void load_v(uint4 (&v)[KK], const DecodeArgs &a, int 
     for (int kk = 0; kk < KK; ++kk) v[kk] = __builtin_bit_cast(uint4, __builtin_nontemporal_load(vp + kk * 64));
 }
 
-template <int P, int WAVES>
+// MQ = false is the decode case (one query row): query slot == head of the group, which
+// spares the integer divisions of the general slot -> (row, head) mapping.
+template <int P, int WAVES, bool MQ>
 __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) {
     constexpr int THREADS = WAVES * 64;
     constexpr int KK = P / 32; // K-steps of the QK product, also column-tile pairs of V
@@ -84,19 +86,19 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     const int j = lane >> 4;
     const int split = blockIdx.x;
     const int kvh = blockIdx.y;
-    const int tile = blockIdx.z;
+    const int tile = MQ ? blockIdx.z : 0;
     const int G = g.gqa;
-    const int C = a.n_queries;
+    const int C = MQ ? a.n_queries : 1;
     const int n_slots = C * G;
     const int rows = min(16, n_slots - tile * 16); // query slots of this workgroup
     // this lane's query slot in the B and D operand layouts
     const int my_slot = min(tile * 16 + n, n_slots - 1);
-    const int my_q = my_slot / G;
+    const int my_q = MQ ? my_slot / G : 0;
     const int my_limit = a.len - C + my_q; // last position the slot attends
     const int my_ws = a.window > 0 ? max(a.window_start, my_limit + 1 - a.window) : a.window_start;
     // extremes over the workgroup's slots
-    const int qrow_lo = (tile * 16) / G;
-    const int qrow_hi = (tile * 16 + rows - 1) / G;
+    const int qrow_lo = MQ ? (tile * 16) / G : 0;
+    const int qrow_hi = MQ ? (tile * 16 + rows - 1) / G : 0;
     const int lim_lo = a.len - C + qrow_lo;
     const int lim_hi = a.len - C + qrow_hi;
     const int ws_lo = a.window > 0 ? max(a.window_start, lim_lo + 1 - a.window) : a.window_start;
@@ -111,8 +113,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     // pages this workgroup's slots can see, divided among the splits
     const int page_lo = g.ring_rows > 0 ? 0 : ws_lo >> 4;
     const int page_hi = g.ring_rows > 0 ? a.n_pages : (lim_hi >> 4) + 1;
-    const int pb0 = page_lo + (int)(((long)split * (page_hi - page_lo)) / a.splits);
-    const int pb1 = page_lo + (int)(((long)(split + 1) * (page_hi - page_lo)) / a.splits);
+    // (32-bit arithmetic: pages * splits stays far below 2^31)
+    const unsigned span = (unsigned)(page_hi - page_lo);
+    const int pb0 = page_lo + (int)(((unsigned)split * span) / (unsigned)a.splits);
+    const int pb1 = page_lo + (int)(((unsigned)(split + 1) * span) / (unsigned)a.splits);
     // this wavefront walks pages pb0 + wave + it * WAVES, it = 0 .. n_it-1
     const int n_it = pb1 - pb0 > wave ? (pb1 - pb0 - wave + WAVES - 1) / WAVES : 0;
 
@@ -160,12 +164,15 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
         const int kk = idx >> 6;
         const int jj = (idx >> 4) & 3;
         const int qs = min(tile * 16 + (idx & 15), n_slots - 1);
-        const float *qrow = a.q + ((long)(qs / G) * g.q_heads + kvh * G + qs % G) * g.head_dim;
+        const float *qrow = a.q + (MQ ? ((long)(qs / G) * g.q_heads + kvh * G + qs % G)
+                                      : (long)(kvh * G + qs)) * g.head_dim;
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[u][e] = qrow[min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
     }
+    // Unconditional (a wavefront without pages reads physical page 0 and ignores it): a
+    // conditional load here makes the compiler wait for these pages before the queries.
     uint4 kr[KK], vr[KK];
-    if (n_it > 0) {
+    {
         const int pg = page_id(0);
         load_k<KK>(kr, a, pg, kvh, lane);
         load_v<KK>(vr, a, pg, kvh, lane);
@@ -373,7 +380,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
         float *dst;
         if (a.splits == 1) {
             acc *= 1.0f / lsum;
-            dst = a.out + ((long)(slot / G) * g.q_heads + kvh * G + slot % G) * g.head_dim + c4;
+            dst = a.out + (MQ ? ((long)(slot / G) * g.q_heads + kvh * G + slot % G)
+                              : (long)(kvh * G + slot)) * g.head_dim + c4;
         } else {
             const long pidx = ((long)kvh * a.splits + split) * n_slots + slot;
             dst = a.part_o + pidx * g.head_dim + c4;
@@ -465,8 +473,8 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
     }
 }
 
-template <int P, int WAVES>
-static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
+template <int P, int WAVES, bool MQ>
+static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     constexpr int KK = P / 32;
     const size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
     const int n_slots = a.n_queries * a.g.gqa;
@@ -476,14 +484,19 @@ static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
     static bool attr_set = false; // per instantiation
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES>),
+            reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES, MQ>),
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
-    hipLaunchKernelGGL((decode_split_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((decode_split_kernel<P, WAVES, MQ>), grid, dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
+}
+
+template <int P, int WAVES>
+static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
+    return a.n_queries > 1 ? launch_split_mq<P, WAVES, true>(a, s) : launch_split_mq<P, WAVES, false>(a, s);
 }
 
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
