@@ -43,6 +43,14 @@ WORKLOADS = {
 }
 
 
+# HBM bytes one attention launch (split + merge) moves, from the hardware counters
+# FETCH_SIZE and WRITE_SIZE collected with rocprofv3 --pmc over this same program and scaled
+# by what the counters read for a copy of known size (the method and the raw readings are in
+# profiles/decode_split_kernel_config2.md). Not measurable from inside this process, so it is
+# a recorded figure, present only for the workload it was taken on.
+MEASURED_TRAFFIC_BYTES = {2: 70202 * 1024}
+
+
 def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> int:
     """Bytes one layer's decode step has to move: K and V once (bf16), q in and ctx out
     (f32), the block table, and the appended row when the append is counted."""
@@ -299,7 +307,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "kernel": "decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
                                "average over the layers)" % (128 if hd <= 128 else 256),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context else None,
                      "bytes_per_launch": launch_bytes,
                      "avg_launch_us": round(kern_avg_us, 2), "median_launch_us": round(kern_med_us, 2)},
     }
