@@ -157,6 +157,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--config", type=int, default=2, choices=sorted(WORKLOADS))
     ap.add_argument("--context", type=int, default=0, help="override the cached rows")
+    ap.add_argument("--batch", type=int, default=1,
+                    help="independent sequences decoded together (configs[4] also asks for 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-restore", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -191,47 +193,66 @@ def main() -> int:
     rng = np.random.default_rng(args.config)
     state = skv.DecodeResidentState(0)
     stream = torch.cuda.current_stream().cuda_stream
-    layers = []
+    B = args.batch
+    if B < 1:
+        print("bench.py: --batch must be at least 1", file=sys.stderr)
+        return 2
+    if B > 1:
+        args.no_cpu_baseline = True   # the CPU sample is one sequence
+    layers = []       # one handle per (layer, sequence), layer-major
     layer_rows = []   # rows each layer attends per step (for the byte count)
     host_kv = []      # first layer's f32 rows, kept for the CPU baseline
     for n, _, _, _, rows, window in groups:
         for _ in range(n):
-            kv = state.full_attention_bf16(rows + 2 * total_steps + 8, qh, kvh, hd, window=window)
-            kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
-            fill = min(rows, window) if window else rows   # a ring only keeps its window
-            k = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
-            v = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
-            kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), fill)
-            torch.cuda.synchronize()
-            if not layers and not args.no_cpu_baseline:
-                host_kv = [k.cpu().numpy(), v.cpu().numpy()]
-            del k, v
-            layers.append(kv)
+            for _ in range(B):   # every sequence owns its pages and its block table
+                kv = state.full_attention_bf16(rows + 2 * total_steps + 8, qh, kvh, hd, window=window)
+                kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+                fill = min(rows, window) if window else rows   # a ring only keeps its window
+                k = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+                v = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+                kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), fill)
+                torch.cuda.synchronize()
+                if not layers and not args.no_cpu_baseline:
+                    host_kv = [k.cpu().numpy(), v.cpu().numpy()]
+                del k, v
+                layers.append(kv)
             layer_rows.append(fill)
 
     n_pass = 2 * total_steps  # timed pass + per-kernel pass
-    q_all = torch.randn(n_pass, layers_n, q_dim, device=dev, dtype=torch.float32, generator=gen)
-    k_all = torch.randn(n_pass, layers_n, kv_dim, device=dev, dtype=torch.float32, generator=gen)
-    v_all = torch.randn(n_pass, layers_n, kv_dim, device=dev, dtype=torch.float32, generator=gen)
-    out = torch.empty(layers_n, q_dim, device=dev, dtype=torch.float32)
+    n_units = layers_n * B   # (layer, sequence) pairs, layer-major
+    q_all = torch.randn(n_pass, n_units, q_dim, device=dev, dtype=torch.float32, generator=gen)
+    k_all = torch.randn(n_pass, n_units, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+    v_all = torch.randn(n_pass, n_units, kv_dim, device=dev, dtype=torch.float32, generator=gen)
+    out = torch.empty(n_units, q_dim, device=dev, dtype=torch.float32)
     torch.cuda.synchronize()
 
     lib = skv.lib()
-    PtrArr = C.c_void_p * layers_n
+    PtrArr = C.c_void_p * n_units
     layer_arr = PtrArr(*[l._h.value for l in layers])
-    out_arr = PtrArr(*[out[i].data_ptr() for i in range(layers_n)])
+    out_arr = PtrArr(*[out[i].data_ptr() for i in range(n_units)])
 
     def ptrs(t, step):
         base, stride = t[step].data_ptr(), t.stride(1) * 4
-        return PtrArr(*[base + i * stride for i in range(layers_n)])
+        return PtrArr(*[base + i * stride for i in range(n_units)])
 
     step_ptrs = [(ptrs(k_all, s), ptrs(v_all, s), ptrs(q_all, s)) for s in range(n_pass)]
+    vpp = C.POINTER(C.c_void_p)
+
+    def at(arr, li):   # the B pointers of layer li inside a layer-major array
+        return C.cast(C.byref(arr, li * B * C.sizeof(C.c_void_p)), vpp)
 
     def run_step(s):
         kp, vp, qp = step_ptrs[s]
-        rc = lib.skv_decode_step_layers_device(layer_arr, layers_n, stream, kp, vp, qp, out_arr)
-        if rc:
-            raise RuntimeError(lib.skv_last_error().decode())
+        if B == 1:
+            rc = lib.skv_decode_step_layers_device(layer_arr, layers_n, stream, kp, vp, qp, out_arr)
+            if rc:
+                raise RuntimeError(lib.skv_last_error().decode())
+            return
+        for li in range(layers_n):   # one launch pair per layer covers the B sequences
+            rc = lib.skv_decode_step_batch_device(at(layer_arr, li), B, stream, at(kp, li), at(vp, li),
+                                                  at(qp, li), at(out_arr, li))
+            if rc:
+                raise RuntimeError(lib.skv_last_error().decode())
 
     for s in range(args.warmup):
         run_step(s)
@@ -242,25 +263,31 @@ def main() -> int:
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    us_per_token = ms_per_step * 1e3
+    step_us = ms_per_step * 1e3
+    us_per_token = step_us / B   # a step yields one token per sequence
     mid = args.warmup + args.steps // 2
-    step_bytes = sum(algorithmic_bytes(min(r + mid, w) if w else r + mid, kv_dim, q_dim, True)
-                     for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
+    step_bytes = B * sum(algorithmic_bytes(min(r + mid, w) if w else r + mid, kv_dim, q_dim, True)
+                         for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
 
     # ---- per-kernel pass on the launch stream: the ten appends of a token first, then HIP
     # events around the ten attention launches (one per layer) so that the cost of recording
     # an event is spread over ten launches
+    # (with a batch the launch is the fused step of the B sequences of one layer)
     evs = []
     for s in range(total_steps, total_steps + args.steps):
         kp, vp, qp = step_ptrs[s]
-        for li, kv in enumerate(layers):
-            kv.encode_append_kv(stream, kp[li], vp[li])
+        if B == 1:
+            for li, kv in enumerate(layers):
+                kv.encode_append_kv(stream, kp[li], vp[li])
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
-        for li, kv in enumerate(layers):
-            ws = max(kv.len() - kv.window(), 0) if kv.window() else 0
-            kv.encode_attention_decode_windowed(stream, qp[li], out_arr[li], ws)
+        if B == 1:
+            for li, kv in enumerate(layers):
+                ws = max(kv.len() - kv.window(), 0) if kv.window() else 0
+                kv.encode_attention_decode_windowed(stream, qp[li], out_arr[li], ws)
+        else:
+            run_step(s)
         e1.record()
         evs.append((e0, e1))
     torch.cuda.synchronize()
@@ -270,8 +297,8 @@ def main() -> int:
     # the dominant launch is a layer of the first group; with mixed groups the event pairs span
     # all layers, so bytes are summed over the layers and divided by the same time
     late = total_steps + args.steps // 2
-    all_bytes = sum(algorithmic_bytes(min(r + late, w) if w else r + late, kv_dim, q_dim, False)
-                    for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
+    all_bytes = B * sum(algorithmic_bytes(min(r + late, w) if w else r + late, kv_dim, q_dim, B > 1)
+                        for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
     launch_bytes = all_bytes // layers_n
     achieved = launch_bytes / (kern_avg_us * 1e-6) / 1e9
     cpu_inputs = None
@@ -298,16 +325,19 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": (wl["name"] % ctx_rows) + ", bf16 KV in 16-token pages, batch 1, "
-                               "1 token per step",
-                   "context": ctx_rows, "layers": layers_n, "page_rows": 16},
+        "config": {"workload": (wl["name"] % ctx_rows) + ", bf16 KV in 16-token pages, batch %d, "
+                               "1 token per sequence per step" % B,
+                   "context": ctx_rows, "layers": layers_n, "page_rows": 16, "batch": B},
         "tok_per_s": round(1e6 / us_per_token, 1),
-        "hbm_gbps": round(step_bytes / (us_per_token * 1e-6) / 1e9, 1),
-        "hbm_frac": round(step_bytes / (us_per_token * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
-                               "average over the layers)" % (128 if hd <= 128 else 256),
+        "hbm_gbps": round(step_bytes / (step_us * 1e-6) / 1e9, 1),
+        "hbm_frac": round(step_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "roofline": {"bound": "hbm", "kernel": ("decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
+                                                "average over the layers)" if B == 1 else
+                                                "decode_split_batch_kernel<%d,8> + decode_merge_batch_kernel (one launch pair "
+                                                "per layer covers the batch, average over the layers)")
+                                               % (128 if hd <= 128 else 256),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context else None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context and B == 1 else None,
                      "bytes_per_launch": launch_bytes,
                      "avg_launch_us": round(kern_avg_us, 2), "median_launch_us": round(kern_med_us, 2)},
     }

@@ -167,6 +167,18 @@ int32_t skv_prefill_chunk_device(skv_layer *layer, skv_stream stream, const floa
 int32_t skv_prefill_chunk_host(skv_layer *layer, const float *q, const float *k, const float *v,
                                size_t n_rows, float *out);
 
+/* One decode step of the SAME model layer for n_seq independent sequences (each its own
+ * handle, block table and length): for sequence i, append k_dev[i]/v_dev[i] (kv_dim f32
+ * each) then attention of q_dev[i] into out_dev[i], all in one pair of launches. The
+ * reference decodes one sequence at a time (encode_resident_full_layer,
+ * src/decode_resident/layers.rs:259-288, once per sequence); this is that call applied to
+ * a batch, with the same result per sequence. All handles must share the head geometry,
+ * the window and the context, and be distinct; nothing is modified when one of them is
+ * at capacity. */
+int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_stream stream,
+                                     const void *const *k_dev, const void *const *v_dev,
+                                     const float *const *q_dev, float *const *out_dev);
+
 /* The KV path of one token over several layers: for each layer i, append
  * k_dev[i]/v_dev[i] (kv_dim f32 each) then attention of q_dev[i] into out_dev[i].
  * It is the per-layer loop of enqueue_decode_token_resident

@@ -85,6 +85,7 @@ SIGNATURES = {
     "skv_decode_step_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp]),
     "skv_prefill_chunk_device": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "skv_prefill_chunk_host": (_i32, [_vp, _vp, _vp, _vp, _sz, _vp]),
+    "skv_decode_step_batch_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_decode_step_layers_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_read_rows": (_i32, [_vp, _sz, _sz, _vp, _vp]),
     "skv_gather_device": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp]),

@@ -70,10 +70,12 @@ __device__ __forceinline__ void load_v(uint4 (&v)[KK], const DecodeArgs &a, int 
     for (int kk = 0; kk < KK; ++kk) v[kk] = __builtin_bit_cast(uint4, __builtin_nontemporal_load(vp + kk * 64));
 }
 
-// MQ = false is the decode case (one query row): query slot == head of the group, which
-// spares the integer divisions of the general slot -> (row, head) mapping.
+// MQ = false is the decode case (one query row, at most 16 heads per group): query slot ==
+// head of the group, which spares the integer divisions of the general slot -> (row, head)
+// mapping.
 template <int P, int WAVES, bool MQ>
-__global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) {
+__device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int split, const int kvh,
+                                                  const int tile_z) {
     constexpr int THREADS = WAVES * 64;
     constexpr int KK = P / 32; // K-steps of the QK product, also column-tile pairs of V
     constexpr int NT = P / 16; // 16-column tiles of the output
@@ -84,9 +86,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15; // key row inside the tile (A operand) / query slot (B, D)
     const int j = lane >> 4;
-    const int split = blockIdx.x;
-    const int kvh = blockIdx.y;
-    const int tile = MQ ? blockIdx.z : 0;
+    const int tile = MQ ? tile_z : 0;
     const int G = g.gqa;
     const int C = MQ ? a.n_queries : 1;
     const int n_slots = C * G;
@@ -402,6 +402,20 @@ __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) 
     }
 }
 
+template <int P, int WAVES, bool MQ>
+__global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) {
+    decode_split_body<P, WAVES, MQ>(a, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// Several independent sequences of the same model layer in one launch: grid z is the
+// sequence, grid x covers the largest split count and the others leave early.
+template <int P, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void decode_split_batch_kernel(DecodeBatchArgs b) {
+    const DecodeArgs &a = b.seq[blockIdx.z];
+    if ((int)blockIdx.x >= a.splits) return;
+    decode_split_body<P, WAVES, false>(a, blockIdx.x, blockIdx.y, 0);
+}
+
 // ------------------------------------------------------------------------------------
 // Merge of the split-K partials: one workgroup per (query head, 16 columns). The 256
 // threads are 16 columns x 16 split lanes. Every thread issues all its loads (o, m, l
@@ -413,7 +427,7 @@ constexpr int MERGE_PER_LANE_MAX = DEC_MAX_SPLITS / 16;
 
 // MERGE_PER_LANE: splits each of the 16 split lanes covers, the smallest power of two that fits
 template <int MERGE_PER_LANE>
-__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
+__device__ __forceinline__ void decode_merge_body(const DecodeArgs &a) {
     const Geom g = a.g;
     const int n_slots = a.n_queries * g.gqa;
     const int kvh = blockIdx.x / n_slots;
@@ -473,6 +487,19 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
     }
 }
 
+template <int MERGE_PER_LANE>
+__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
+    decode_merge_body<MERGE_PER_LANE>(a);
+}
+
+// grid z is the sequence; a sequence with a single split already has its context
+template <int MERGE_PER_LANE>
+__global__ __launch_bounds__(256) void decode_merge_batch_kernel(DecodeBatchArgs b) {
+    const DecodeArgs &a = b.seq[blockIdx.z];
+    if (a.splits <= 1) return;
+    decode_merge_body<MERGE_PER_LANE>(a);
+}
+
 template <int P, int WAVES, bool MQ>
 static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     constexpr int KK = P / 32;
@@ -496,7 +523,9 @@ static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
 
 template <int P, int WAVES>
 static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
-    return a.n_queries > 1 ? launch_split_mq<P, WAVES, true>(a, s) : launch_split_mq<P, WAVES, false>(a, s);
+    // the decode specialisation assumes a single tile of query slots
+    return a.n_queries > 1 || a.g.gqa > 16 ? launch_split_mq<P, WAVES, true>(a, s)
+                                           : launch_split_mq<P, WAVES, false>(a, s);
 }
 
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
@@ -518,6 +547,55 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     else if (per_lane <= 8) hipLaunchKernelGGL(decode_merge_kernel<8>, mgrid, dim3(256), 0, s, a);
     else if (per_lane <= 16) hipLaunchKernelGGL(decode_merge_kernel<16>, mgrid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL(decode_merge_kernel<MERGE_PER_LANE_MAX>, mgrid, dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+template <int P, int WAVES>
+static hipError_t launch_split_batch(const DecodeBatchArgs &b, int n_seq, int max_splits, hipStream_t s) {
+    constexpr int KK = P / 32;
+    const Geom &g = b.seq[0].g;
+    const size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
+    const int rows = g.gqa < 16 ? g.gqa : 16;
+    const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
+    const size_t lds = stage > xchg ? stage : xchg;
+    static bool attr_set = false; // per instantiation
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&decode_split_batch_kernel<P, WAVES>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    dim3 grid((unsigned)max_splits, (unsigned)g.kv_heads, (unsigned)n_seq);
+    hipLaunchKernelGGL((decode_split_batch_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, b);
+    return hipGetLastError();
+}
+
+// All sequences share one geometry and one wavefront count, and each has n_queries == 1
+// and gqa <= 16 (checked by the caller).
+hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s) {
+    if (n_seq < 1 || n_seq > SKV_MAX_BATCH) return hipErrorInvalidValue;
+    const DecodeArgs &a0 = b.seq[0];
+    int max_splits = 1;
+    for (int i = 0; i < n_seq; ++i) max_splits = b.seq[i].splits > max_splits ? b.seq[i].splits : max_splits;
+    hipError_t e = hipErrorInvalidValue;
+    const bool w8 = a0.waves == 8;
+    switch (a0.g.P) {
+    case 32: e = w8 ? launch_split_batch<32, 8>(b, n_seq, max_splits, s) : launch_split_batch<32, 4>(b, n_seq, max_splits, s); break;
+    case 64: e = w8 ? launch_split_batch<64, 8>(b, n_seq, max_splits, s) : launch_split_batch<64, 4>(b, n_seq, max_splits, s); break;
+    case 128: e = w8 ? launch_split_batch<128, 8>(b, n_seq, max_splits, s) : launch_split_batch<128, 4>(b, n_seq, max_splits, s); break;
+    case 256: e = w8 ? launch_split_batch<256, 8>(b, n_seq, max_splits, s) : launch_split_batch<256, 4>(b, n_seq, max_splits, s); break;
+    default: break;
+    }
+    if (e != hipSuccess || max_splits == 1) return e;
+    dim3 mgrid((unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)((a0.g.head_dim + 15) / 16), (unsigned)n_seq);
+    const int per_lane = (max_splits + 15) / 16;
+    if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_batch_kernel<1>, mgrid, dim3(256), 0, s, b);
+    else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_batch_kernel<2>, mgrid, dim3(256), 0, s, b);
+    else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_batch_kernel<4>, mgrid, dim3(256), 0, s, b);
+    else if (per_lane <= 8) hipLaunchKernelGGL(decode_merge_batch_kernel<8>, mgrid, dim3(256), 0, s, b);
+    else if (per_lane <= 16) hipLaunchKernelGGL(decode_merge_batch_kernel<16>, mgrid, dim3(256), 0, s, b);
+    else hipLaunchKernelGGL(decode_merge_batch_kernel<MERGE_PER_LANE_MAX>, mgrid, dim3(256), 0, s, b);
     return hipGetLastError();
 }
 

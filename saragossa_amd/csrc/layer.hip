@@ -63,9 +63,10 @@ int choose_waves(const skv_layer *L) {
     return w == 4 ? 4 : 8;
 }
 
-int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows, int waves) {
+size_t decode_target_wgs() { return std::max<size_t>(env_usize("SKV_DECODE_WGS", 256), 1); }
+
+int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows, int waves, size_t target_wgs) {
     if (!skv_flag_sdpa_2pass_enabled() || rows < split_min_len()) return 1;
-    const size_t target_wgs = env_usize("SKV_DECODE_WGS", 256);
     const size_t min_pages = std::max<size_t>(env_usize("SKV_DECODE_MIN_PAGES", (size_t)waves), 1);
     size_t s = std::max<size_t>(target_wgs / (size_t)L->g.kv_heads, 1);
     s = std::min<size_t>(s, (size_t)n_pages_scan / min_pages);
@@ -89,6 +90,45 @@ int32_t check_window(const skv_layer *L, size_t window_start) {
 }
 
 bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L->g.P <= 256; }
+
+// Arguments of the matrix-core attention kernel for the layer's current length.
+void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, size_t window_start,
+                      const float *k_new, const float *v_new, size_t n_queries, size_t target_wgs,
+                      DecodeArgs &a) {
+    const Geom &g = L->g;
+    a.q = q_dev;
+    a.out = out_dev;
+    a.k_pool = L->k_pool;
+    a.v_pool = L->v_pool;
+    a.table = L->table_dev;
+    a.part_o = L->part_o;
+    a.part_m = L->part_m;
+    a.part_l = L->part_l;
+    a.len = (int)L->len;
+    a.n_queries = (int)n_queries;
+    a.window = n_queries > 1 ? (int)L->window : 0; // decode callers pass window_start themselves
+    a.window_start = (int)window_start;
+    if (g.ring_rows > 0) {
+        a.page_first = 0;
+        a.n_pages = (int)std::min<size_t>((L->len + 15) / 16, (size_t)L->n_pages);
+        a.ring_t = (int)((L->len - 1) % (size_t)g.ring_rows);
+        a.ring_base = (int)(L->len - 1) - a.ring_t;
+    } else {
+        a.page_first = (int)(window_start / 16);
+        a.n_pages = (int)((L->len + 15) / 16) - a.page_first;
+    }
+    a.waves = choose_waves(L);
+    a.splits = choose_splits(L, a.n_pages, L->len - window_start, a.waves, target_wgs);
+    // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
+    // 575); log2(e) moves the softmax to base 2.
+    a.qscale = (1.0f / std::sqrt((float)g.head_dim)) * 1.4426950408889634f;
+    a.k_new = k_new;
+    a.v_new = v_new;
+    a.k_pool_w = L->k_pool;
+    a.v_pool_w = L->v_pool;
+    a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
+    a.g = g;
+}
 
 // k_new / v_new non-null: the row at position len-1 has not been written yet and the
 // attention kernel appends it itself (the host bookkeeping has already advanced).
@@ -129,29 +169,7 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
         return SKV_OK;
     }
     DecodeArgs a{};
-    a.q = q_dev;
-    a.out = out_dev;
-    a.k_pool = L->k_pool;
-    a.v_pool = L->v_pool;
-    a.table = L->table_dev;
-    a.part_o = L->part_o;
-    a.part_m = L->part_m;
-    a.part_l = L->part_l;
-    a.len = (int)L->len;
-    a.n_queries = (int)n_queries;
-    a.window = n_queries > 1 ? (int)L->window : 0; // decode callers pass window_start themselves
-    a.window_start = (int)window_start;
-    if (g.ring_rows > 0) {
-        a.page_first = 0;
-        a.n_pages = (int)std::min<size_t>((L->len + 15) / 16, (size_t)L->n_pages);
-        a.ring_t = (int)((L->len - 1) % (size_t)g.ring_rows);
-        a.ring_base = (int)(L->len - 1) - a.ring_t;
-    } else {
-        a.page_first = (int)(window_start / 16);
-        a.n_pages = (int)((L->len + 15) / 16) - a.page_first;
-    }
-    a.waves = choose_waves(L);
-    a.splits = choose_splits(L, a.n_pages, L->len - window_start, a.waves);
+    fill_decode_args(L, q_dev, out_dev, window_start, k_new, v_new, n_queries, decode_target_wgs(), a);
     if (n_queries > 1) {
         // every 16 query slots are a workgroup of their own: split the context only while
         // that leaves compute units idle, and keep the partials in the context's scratch
@@ -175,15 +193,6 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
             a.part_l = a.part_m + n_part;
         }
     }
-    // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
-    // 575); log2(e) moves the softmax to base 2.
-    a.qscale = (1.0f / std::sqrt((float)g.head_dim)) * 1.4426950408889634f;
-    a.k_new = k_new;
-    a.v_new = v_new;
-    a.k_pool_w = L->k_pool;
-    a.v_pool_w = L->v_pool;
-    a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
-    a.g = g;
     SKV_HIP(launch_decode(a, s));
     return SKV_OK;
 }
@@ -286,8 +295,6 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
         return fail(SKV_ERR_CONFIG, "KV f32 non construit dans cette bibliothèque: bf16 uniquement");
     const int P = padded_head_dim(head_dim);
     if (P == 0) return fail(SKV_ERR_CONFIG, "head_dim > 512 non supporté");
-    if (q_heads / kv_heads > 16)
-        return fail(SKV_ERR_CONFIG, "groupe GQA > 16 non supporté");
     if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096)
         return fail(SKV_ERR_CONFIG, "capacité KV déborde");
     SKV_HIP(hipSetDevice(ctx->device));
@@ -580,6 +587,71 @@ int32_t skv_prefill_chunk_host(skv_layer *L, const float *q, const float *k, con
     if (e != hipSuccess) return fail_hip(e, "prefill chunk: copie");
     if (rc) return rc;
     if (e2 != hipSuccess) return fail_hip(e2, "prefill chunk: synchronisation");
+    return SKV_OK;
+}
+
+int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_stream stream,
+                                     const void *const *k_dev, const void *const *v_dev,
+                                     const float *const *q_dev, float *const *out_dev) {
+    if (!seqs || !k_dev || !v_dev || !q_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step_batch: pointeur nul");
+    if (n_seq == 0) return fail(SKV_ERR_DIMENSION, "decode_step_batch: aucune séquence");
+    for (size_t i = 0; i < n_seq; ++i) {
+        const skv_layer *L = seqs[i];
+        if (!L || !k_dev[i] || !v_dev[i] || !q_dev[i] || !out_dev[i])
+            return fail(SKV_ERR_DEVICE, "decode_step_batch: pointeur nul (séquence " + std::to_string(i) + ")");
+        const Geom &g = L->g, &g0 = seqs[0]->g;
+        if (g.q_heads != g0.q_heads || g.kv_heads != g0.kv_heads || g.head_dim != g0.head_dim ||
+            g.ring_rows != g0.ring_rows || L->window != seqs[0]->window || L->ctx != seqs[0]->ctx)
+            return fail(SKV_ERR_DIMENSION, "decode_step_batch: la séquence " + std::to_string(i) +
+                                               " n'a pas la géométrie de la séquence 0");
+        for (size_t j = 0; j < i; ++j)
+            if (seqs[j] == L)
+                return fail(SKV_ERR_DIMENSION, "decode_step_batch: séquence " + std::to_string(i) + " en double");
+        // nothing is modified unless every sequence can take its row
+        if (L->len >= L->capacity)
+            return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " + std::to_string(L->capacity) +
+                                               " atteinte (overflow), séquence " + std::to_string(i));
+    }
+    static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
+    if (!fused || !uses_flash(seqs[0]) || seqs[0]->g.gqa > 16 || n_seq == 1) {
+        for (size_t i = 0; i < n_seq; ++i) {
+            int32_t rc = skv_decode_step_device(seqs[i], stream, k_dev[i], 0, v_dev[i], 0, q_dev[i], out_dev[i]);
+            if (rc) return rc;
+        }
+        return SKV_OK;
+    }
+    for (size_t first = 0; first < n_seq; first += SKV_MAX_BATCH) {
+        const size_t n = std::min<size_t>(SKV_MAX_BATCH, n_seq - first);
+        // the workgroup budget is shared in proportion to the pages each sequence scans
+        size_t pages_total = 0;
+        for (size_t i = 0; i < n; ++i) {
+            const skv_layer *L = seqs[first + i];
+            const size_t rows = L->g.ring_rows > 0 ? std::min<size_t>(L->len + 1, (size_t)L->g.ring_rows)
+                                                   : L->len + 1 - skv_window_start(L->len, L->window);
+            pages_total += (rows + 15) / 16;
+        }
+        DecodeBatchArgs b{};
+        for (size_t i = 0; i < n; ++i) {
+            skv_layer *L = seqs[first + i];
+            // the attention kernel writes the row itself: advance the bookkeeping first
+            L->len += 1;
+            if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
+                L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
+            const size_t ws = skv_window_start(L->len - 1, L->window);
+            const size_t rows = L->g.ring_rows > 0 ? std::min<size_t>(L->len, (size_t)L->g.ring_rows) : L->len - ws;
+            const size_t share = std::max<size_t>(decode_target_wgs() * ((rows + 15) / 16) / std::max<size_t>(pages_total, 1),
+                                                  (size_t)L->g.kv_heads);
+            fill_decode_args(L, q_dev[first + i], out_dev[first + i], ws,
+                             reinterpret_cast<const float *>(k_dev[first + i]),
+                             reinterpret_cast<const float *>(v_dev[first + i]), 1, share, b.seq[i]);
+        }
+        hipError_t e = launch_decode_batch(b, (int)n, as_stream(stream));
+        if (e != hipSuccess) {
+            for (size_t i = 0; i < n; ++i) seqs[first + i]->len -= 1;
+            return fail_hip(e, "decode_step_batch: lancement");
+        }
+    }
     return SKV_OK;
 }
 

@@ -112,6 +112,13 @@ struct DecodeArgs {
     Geom g;
 };
 
+// One decode step of the same model layer for several independent sequences.
+constexpr int SKV_MAX_BATCH = 16;
+struct DecodeBatchArgs {
+    DecodeArgs seq[SKV_MAX_BATCH];
+};
+static_assert(sizeof(DecodeBatchArgs) <= 4096, "kernel arguments are limited to 4 KiB");
+
 struct NaiveArgs {
     const float *q;
     float *out;
@@ -129,6 +136,7 @@ struct NaiveArgs {
 hipError_t launch_append(const AppendArgs &a, hipStream_t s);
 hipError_t launch_gather(const GatherArgs &a, hipStream_t s);
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s);
+hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s);
 hipError_t launch_naive(const NaiveArgs &a, hipStream_t s);
 int decode_max_splits();
 

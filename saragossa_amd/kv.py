@@ -174,3 +174,21 @@ class FullAttentionState:
 
     def encode_gather(self, stream, first, n, k_dst_ptr, v_dst_ptr) -> None:
         check(self._l.skv_gather_device(self._h, stream, first, n, k_dst_ptr, v_dst_ptr))
+
+
+def encode_decode_step_batch(seqs, stream, k_ptrs, v_ptrs, q_ptrs, out_ptrs) -> None:
+    """One decode step of the same model layer for several independent sequences in one pair
+    of launches (skv_decode_step_batch_device): sequence i appends the kv_dim f32 values at
+    k_ptrs[i] / v_ptrs[i], then attends q_ptrs[i] into out_ptrs[i]. Per sequence it is
+    FullAttentionState.encode_decode_step (src/decode_resident/layers.rs:259-288)."""
+    import ctypes as C
+    n = len(seqs)
+    if not (len(k_ptrs) == len(v_ptrs) == len(q_ptrs) == len(out_ptrs) == n):
+        raise ValueError("one k, v, q and out pointer per sequence")
+    arr = C.c_void_p * n
+    l = seqs[0]._l if n else None
+    if l is None:
+        from ._lib import lib
+        l = lib()
+    check(l.skv_decode_step_batch_device(arr(*[s._h for s in seqs]), n, stream, arr(*k_ptrs),
+                                         arr(*v_ptrs), arr(*q_ptrs), arr(*out_ptrs)))

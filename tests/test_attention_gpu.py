@@ -62,7 +62,8 @@ def test_attention_decode_2pass_d128_matches_cpu(state, n):
 
 
 @pytest.mark.parametrize("dims", [(4, 2, 16), (4, 4, 64), (8, 1, 32), (6, 2, 96), (2, 1, 40),
-                                  (32, 8, 128), (16, 8, 256), (32, 2, 128)])
+                                  (32, 8, 128), (16, 8, 256), (32, 2, 128),
+                                  (40, 1, 64), (48, 2, 32)])   # the last two: more than 16 heads per group
 @pytest.mark.parametrize("n", [3, 100, 1500])
 def test_attention_decode_other_shapes(state, dims, n):
     run_attention_case(state, n, *dims)

@@ -150,3 +150,94 @@ def test_ring_layer_host_api(state):
         kv.read_rows(0, 4)
     gk, _ = kv.read_rows_f32(n - window, window)
     assert np.array_equal(gk, cache.keys()[n - window:])
+
+
+@pytest.mark.parametrize("dims,window,starts,steps", [
+    ((16, 8, 256), 0, [4100, 33, 900, 0], 24),     # config 4's global shape: long, short (one split), empty
+    ((16, 8, 256), 64, [500, 0, 70, 63], 40),      # ring layers at different fill levels and wraps
+    ((32, 8, 128), 0, [260, 2000], 20),            # two sequences, Qwen3-4B shape
+    ((8, 2, 64), 0, list(range(100, 1900, 100)), 6),  # 18 sequences: more than one launch's worth
+])
+def test_decode_step_batch_matches_oracle(state, dims, window, starts, steps):
+    """A batch of independent sequences through skv_decode_step_batch_device: every sequence
+    gets what its own append + cached_attention_one gives (same bound as the single-sequence
+    step), contents stay bit-exact, and the batch agrees with single-sequence calls."""
+    q_heads, kv_heads, head_dim = dims
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(len(starts) * 1000 + steps)
+    n = len(starts)
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    seqs, twins, caches = [], [], []
+    for start in starts:
+        cap = start + steps
+        kv = state.full_attention_bf16(cap, q_heads, kv_heads, head_dim, window=window)
+        kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+        twin = state.full_attention_bf16(cap, q_heads, kv_heads, head_dim, window=window)
+        cache = oracle.LayerKvCache("bf16r")
+        if start:
+            k0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+            v0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+            kv.seed(k0, v0, start)
+            twin.seed(k0, v0, start)
+            cache.append_batch(k0, v0, lay)
+        seqs.append(kv)
+        twins.append(twin)
+        caches.append(cache)
+    ks = rng.standard_normal((steps, n, kv_dim), dtype=np.float32)
+    vs = rng.standard_normal((steps, n, kv_dim), dtype=np.float32)
+    qs = rng.standard_normal((steps, n, q_dim), dtype=np.float32)
+    kd, vd, qd = _dev(ks), _dev(vs), _dev(qs)
+    out = torch.empty(steps, n, q_dim, device="cuda", dtype=torch.float32)
+    single = torch.empty(steps, n, q_dim, device="cuda", dtype=torch.float32)
+    for t in range(steps):
+        skv.encode_decode_step_batch(
+            seqs, _stream(), [kd[t, i].data_ptr() for i in range(n)],
+            [vd[t, i].data_ptr() for i in range(n)], [qd[t, i].data_ptr() for i in range(n)],
+            [out[t, i].data_ptr() for i in range(n)])
+        for i in range(n):
+            twins[i].encode_decode_step(_stream(), kd[t, i].data_ptr(), 0, vd[t, i].data_ptr(), 0,
+                                        qd[t, i].data_ptr(), single[t, i].data_ptr())
+    got, one = out.cpu().numpy(), single.cpu().numpy()
+    # the two differ only in how many splits the context was cut into
+    assert np.abs(got - one).max() <= 2e-6
+    worst = 0.0
+    for i in range(n):
+        for t in range(steps):
+            want = oracle.decode_step(caches[i], ks[t, i], vs[t, i], qs[t, i], lay)
+            worst = max(worst, float(np.abs(got[t, i] - want).max()))
+    assert worst <= 1e-4, worst
+    for i, start in enumerate(starts):
+        cap = start + steps
+        assert seqs[i].len() == cap
+        first = 0 if window == 0 else max(0, cap - (window + 15) // 16 * 16)
+        gk, gv = seqs[i].read_rows_f32(first, cap - first)
+        assert np.array_equal(gk, caches[i].keys()[first:])
+        assert np.array_equal(gv, caches[i].values()[first:])
+
+
+def test_decode_step_batch_errors(state):
+    """Mixed geometries, a repeated handle and a full sequence are errors, and a failed call
+    leaves every sequence as it was."""
+    a = state.full_attention_bf16(40, 8, 2, 64)
+    b = state.full_attention_bf16(40, 8, 2, 64)
+    c = state.full_attention_bf16(40, 8, 4, 64)
+    full = state.full_attention_bf16(4, 8, 2, 64)
+    z = np.zeros((4, 2 * 64), np.float32)
+    full.seed(z, z, 4)
+    buf = torch.zeros(8 * 64, device="cuda", dtype=torch.float32)
+    p = buf.data_ptr()
+    with pytest.raises(skv.DimensionError):
+        skv.encode_decode_step_batch([a, c], _stream(), [p, p], [p, p], [p, p], [p, p])
+    with pytest.raises(skv.DimensionError):
+        skv.encode_decode_step_batch([a, a], _stream(), [p, p], [p, p], [p, p], [p, p])
+    with pytest.raises(skv.DimensionError):
+        skv.encode_decode_step_batch([a, b, full], _stream(), [p] * 3, [p] * 3, [p] * 3, [p] * 3)
+    with pytest.raises(skv.DeviceError):
+        skv.encode_decode_step_batch([a, b], _stream(), [p, 0], [p, p], [p, p], [p, p])
+    assert a.len() == 0 and b.len() == 0 and full.len() == 4
+    out = torch.empty(2, 8 * 64, device="cuda", dtype=torch.float32)
+    skv.encode_decode_step_batch([a, b], _stream(), [p, p], [p, p], [p, p],
+                                 [out[0].data_ptr(), out[1].data_ptr()])
+    torch.cuda.synchronize()
+    assert a.len() == 1 and b.len() == 1
+    assert np.array_equal(out.cpu().numpy(), np.zeros((2, 8 * 64), np.float32))  # one key: out == its V row
