@@ -167,6 +167,52 @@ int32_t skv_prefill_chunk_device(skv_layer *layer, skv_stream stream, const floa
 int32_t skv_prefill_chunk_host(skv_layer *layer, const float *q, const float *k, const float *v,
                                size_t n_rows, float *out);
 
+/* ---- The step before the cache: per-head RMSNorm + rotation at the token's position ----
+ * rope_rotations (src/decoder/attention_ops.rs:848-887): cos and sin of
+ * (position * position_scale) / theta^(2*pair / frequency_dim) for every pair, computed
+ * on the host in f32 with libm exactly as the reference's CPU path does; cos_sin_out
+ * receives rope_dims floats, (cos, sin) per pair. frequency_dim 0 = rope_dims. */
+int32_t skv_rope_rotations_host(size_t position, size_t rope_dims, size_t frequency_dim, float theta,
+                                float position_scale, float *cos_sin_out);
+
+/* The same rotations for positions 0..max_positions-1 as a device table, built once per
+ * (theta, scale, rope_dims) of a model; it replaces the reference's process-global memo of
+ * rope_rotations. style: 0 = RopeStyle::Halves, 1 = RopeStyle::Interleaved
+ * (src/decoder.rs:70-76). */
+typedef struct skv_rope skv_rope;
+int32_t skv_rope_create(skv_ctx *ctx, size_t max_positions, size_t rope_dims, size_t frequency_dim,
+                        float theta, float position_scale, int32_t style, skv_rope **out);
+void skv_rope_destroy(skv_rope *rope);
+
+/* encode_rms_norm_rope_decode[_with_offset] (src/decode_resident/layers.rs:214-227, kernel
+ * rms_norm_rope_heads_decode_f32, src/decode_resident/kernels.rs:975-1027): out = per-head
+ * RMSNorm(x) * weight, then the rotation of `position` on the first rope_dims dims of each
+ * head. weight_dev null = no norm (apply_rope_heads_at, attention_ops.rs:779-834); rope
+ * null = no rotation. Same arithmetic, in the same order, as rms_norm_rope_heads_at
+ * (attention_ops.rs:682-777). */
+int32_t skv_rms_norm_rope_decode_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
+                                        size_t position, const float *x_dev, const float *weight_dev,
+                                        size_t heads, size_t head_dim, float eps, float *out_dev);
+/* DecodeResidentState::rms_norm_rope_decode (src/decode_resident/tests.rs:1168-1172, 1883):
+ * host in, host out, synchronous; the rotations of `position` are computed on the host. */
+int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float *weight, size_t heads,
+                                      size_t head_dim, size_t rope_dims, size_t frequency_dim,
+                                      size_t position, float eps, float theta, float position_scale,
+                                      int32_t style, float *out);
+
+/* encode_resident_full_layer from the q/k norms to the attention context
+ * (src/decode_resident/layers.rs:214-288) in one launch pair: RMSNorm + rotation of the raw
+ * q (q_heads*head_dim f32 at q_dev + q_off) and of the raw k row, the query scale
+ * sqrt(head_dim / attn_scalar) (encode_query_attention_scale, layers.rs:7-33; an invalid
+ * attn_scalar is SKV_ERR_CONFIG), append of (k, v) and attention through the layer's
+ * window. q_norm_w / k_norm_w: device f32[head_dim], null = that norm is skipped. The
+ * finished q is not written back; the appended k row is the CPU path's row bit for bit. */
+int32_t skv_decode_step_prekv_device(skv_layer *layer, skv_stream stream, const skv_rope *rope,
+                                     size_t position, const void *q_dev, size_t q_off,
+                                     const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
+                                     const float *q_norm_w, const float *k_norm_w, float eps,
+                                     float attn_scalar, float *out_dev);
+
 /* One decode step of the SAME model layer for n_seq independent sequences (each its own
  * handle, block table and length): for sequence i, append k_dev[i]/v_dev[i] (kv_dim f32
  * each) then attention of q_dev[i] into out_dev[i], all in one pair of launches. The

@@ -117,6 +117,8 @@ hipError_t launch_gather(const GatherArgs &a, hipStream_t s) {
 // RETI_RUST_FLASH_SDPA=0 and serves as an independent check of the matrix-core kernel.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void naive_kernel(NaiveArgs a) {
+    // the __f*_rn intrinsics are plain operators here: without this they fuse into FMAs
+#pragma clang fp contract(off)
     const Geom g = a.g;
     const int h = blockIdx.x;
     const int kvh = h / g.gqa;
@@ -177,6 +179,41 @@ __global__ __launch_bounds__(256) void naive_kernel(NaiveArgs a) {
 
 hipError_t launch_naive(const NaiveArgs &a, hipStream_t s) {
     hipLaunchKernelGGL(naive_kernel, dim3((unsigned)a.g.q_heads), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------
+// Per-head RMSNorm + rotation of one row, one workgroup per head
+// (rms_norm_rope_heads_decode_f32, src/decode_resident/kernels.rs:975-1027). The sum of
+// squares is taken in index order by one lane, like the CPU path, so the row is the CPU
+// row bit for bit.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void norm_rope_kernel(NormRopeArgs a) {
+    __shared__ float row[512];
+    __shared__ float w[512];
+    __shared__ float rope[512];
+    __shared__ float inv_s;
+    const int head = blockIdx.x;
+    const int tid = threadIdx.x;
+    const float *x = a.x + (long)head * a.head_dim;
+    for (int c = tid; c < a.head_dim; c += 256) {
+        row[c] = x[c];
+        w[c] = a.weight ? a.weight[c] : 1.0f;
+        rope[c] = (a.rope && c < a.rope_dims) ? a.rope[c] : 0.0f;
+    }
+    __syncthreads();
+    if (tid == 0) inv_s = a.weight ? head_inv_rms(row, a.head_dim, a.eps) : 1.0f;
+    __syncthreads();
+    const float inv = inv_s;
+    for (int c = tid; c < a.head_dim; c += 256)
+        a.out[(long)head * a.head_dim + c] =
+            norm_rope_elem(row, c, inv, a.weight ? w : nullptr, a.rope ? rope : nullptr, a.rope_dims,
+                           a.rope_style);
+}
+
+hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s) {
+    if (a.heads <= 0 || a.head_dim <= 0 || a.head_dim > 512) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(norm_rope_kernel, dim3((unsigned)a.heads), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -73,7 +73,10 @@ __device__ __forceinline__ void load_v(uint4 (&v)[KK], const DecodeArgs &a, int 
 // MQ = false is the decode case (one query row, at most 16 heads per group): query slot ==
 // head of the group, which spares the integer divisions of the general slot -> (row, head)
 // mapping.
-template <int P, int WAVES, bool MQ>
+// PRE = true fuses the step before the cache (decode only): q and the appended k row arrive
+// raw, and every workgroup applies the per-head RMSNorm and the rotation of the position to
+// the rows it uses, in LDS, while its first page is in flight.
+template <int P, int WAVES, bool MQ, bool PRE>
 __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int split, const int kvh,
                                                   const int tile_z) {
     constexpr int THREADS = WAVES * 64;
@@ -109,6 +112,17 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     uint4 *q_lo = smem + KK * 64;
     uint16_t *new_k = reinterpret_cast<uint16_t *>(smem + 2 * KK * 64); // [P] appended row
     uint16_t *new_v = new_k + P;
+    // PRE: raw and finished rows of the group's queries plus the new k row, weights, rotation
+    constexpr int PS = P + 1;      // row stride: lanes walking different rows hit different banks
+    constexpr int PRE_ROWS = 17;   // 16 query slots + the k row
+    float *pre_raw = reinterpret_cast<float *>(new_v + P); // [PRE_ROWS][PS]
+    float *pre_out = pre_raw + PRE_ROWS * PS;              // [PRE_ROWS][PS]
+    float *pre_wq = pre_out + PRE_ROWS * PS;               // [P]
+    float *pre_wk = pre_wq + P;                            // [P]
+    float *pre_rope = pre_wk + P;                          // [P]: (cos, sin) pairs
+    float *pre_inv = pre_rope + P;                         // [PRE_ROWS] (+5 keeps pre_sq 16-byte aligned)
+    constexpr int SQS = P + 4;                             // 16-byte aligned rows, conflict-free
+    float *pre_sq = pre_inv + PRE_ROWS + 5;                // [PRE_ROWS][SQS]: squares, zero padded
 
     // pages this workgroup's slots can see, divided among the splits
     const int page_lo = g.ring_rows > 0 ? 0 : ws_lo >> 4;
@@ -123,24 +137,31 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     // Fused append: the workgroup whose range holds the page of the new row rounds that
     // row to bf16, stores it into the pools for later steps and keeps it in LDS; the
     // wavefront that walks the page patches its registers from there, so nothing is read
-    // back from memory in this launch.
+    // back from memory in this launch. The row is fetched here, ahead of the pages.
     const int pb_new = a.new_slot >> 4;
     const int r_new = a.new_slot & 15;
     const bool appends = a.k_new != nullptr && C == 1 && pb_new >= pb0 && pb_new < pb1;
-    if (appends) {
-        const int page = a.table[pb_new];
-        const long tile = (long)page * g.page_elems + (long)kvh * g.tile_elems;
-        for (int d = tid; d < P; d += THREADS) {
-            uint16_t kb = 0, vb = 0;
-            if (d < g.head_dim) {
-                kb = bf16_bits(a.k_new[kvh * g.head_dim + d]);
-                vb = bf16_bits(a.v_new[kvh * g.head_dim + d]);
-                a.k_pool_w[tile + k_index(P, r_new, d)] = kb;
-                a.v_pool_w[tile + v_index(P, r_new, d)] = vb;
-            }
-            new_k[d] = kb;
-            new_v[d] = vb;
+    float k_row = 0.0f, v_row = 0.0f; // element tid of the new row of this kv head
+    if (appends && tid < g.head_dim) {
+        k_row = a.k_new[kvh * g.head_dim + tid];
+        v_row = a.v_new[kvh * g.head_dim + tid];
+    }
+    // PRE: raw query rows of the group (and the raw k row, already in k_row)
+    constexpr int PRE_U = PRE ? (16 * P + THREADS - 1) / THREADS : 1;
+    float pre_q[PRE_U];
+    float pre_w0 = 1.0f, pre_w1 = 1.0f, pre_r = 0.0f;
+    if (PRE) {
+#pragma unroll
+        for (int u = 0; u < PRE_U; ++u) {
+            const int e = tid + u * THREADS;
+            const int r = e / P, c = e % P;
+            pre_q[u] = (r < rows && c < g.head_dim) ? a.q[(long)(kvh * G + r) * g.head_dim + c] : 0.0f;
         }
+        if (tid < g.head_dim) {
+            if (a.q_norm_w) pre_w0 = a.q_norm_w[tid];
+            if (a.k_norm_w) pre_w1 = a.k_norm_w[tid];
+        }
+        if (a.rope && tid < a.rope_dims) pre_r = a.rope[tid];
     }
 
     // Block-table entries of the next 64 iterations, one per lane.
@@ -159,7 +180,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     constexpr int QI = (KK * 64 + THREADS - 1) / THREADS;
     float qv[QI][8];
 #pragma unroll
-    for (int u = 0; u < QI; ++u) {
+    for (int u = 0; u < (PRE ? 0 : QI); ++u) {
         const int idx = min(tid + u * THREADS, KK * 64 - 1);
         const int kk = idx >> 6;
         const int jj = (idx >> 4) & 3;
@@ -176,6 +197,76 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         const int pg = page_id(0);
         load_k<KK>(kr, a, pg, kvh, lane);
         load_v<KK>(vr, a, pg, kvh, lane);
+    }
+    if (PRE) {
+        auto sq_of = [](float x) {
+#pragma clang fp contract(off)
+            return x * x;
+        };
+        // rows 0..rows-1: the group's queries; row `rows`: the new k row (appending workgroup)
+#pragma unroll
+        for (int u = 0; u < PRE_U; ++u) {
+            const int e = tid + u * THREADS;
+            const int r = e / P, c = e % P;
+            if (r < rows) {
+                pre_raw[r * PS + c] = pre_q[u];
+                pre_sq[r * SQS + c] = sq_of(pre_q[u]);
+            }
+        }
+        if (tid < P) {
+            pre_raw[rows * PS + tid] = k_row;
+            pre_sq[rows * SQS + tid] = sq_of(k_row);
+            pre_wq[tid] = pre_w0;
+            pre_wk[tid] = pre_w1;
+            pre_rope[tid] = pre_r;
+        }
+        __syncthreads();
+        const int n_rows = rows + (appends ? 1 : 0);
+        if (tid < n_rows) {
+            const bool is_k = tid == rows;
+            const bool has_norm = is_k ? a.k_norm_w != nullptr : a.q_norm_w != nullptr;
+            pre_inv[tid] = has_norm ? head_inv_rms_sq(pre_sq + tid * SQS, P, g.head_dim, a.eps) : 1.0f;
+        }
+        __syncthreads();
+        const float *rope = a.rope ? pre_rope : nullptr;
+        for (int e = tid; e < n_rows * P; e += THREADS) {
+            const int r = e / P, c = e % P;
+            if (c < g.head_dim) {
+                const bool is_k = r == rows;
+                const float *w = is_k ? (a.k_norm_w ? pre_wk : nullptr) : (a.q_norm_w ? pre_wq : nullptr);
+                pre_out[r * PS + c] = norm_rope_elem(pre_raw + r * PS, c, pre_inv[r], w, rope,
+                                                     a.rope_dims, a.rope_style);
+            }
+        }
+        __syncthreads();
+        if (appends && tid < g.head_dim) k_row = pre_out[rows * PS + tid];
+    }
+    if (appends) {
+        const int page = a.table[pb_new];
+        const long tile_at = (long)page * g.page_elems + (long)kvh * g.tile_elems;
+        if (tid < P) {
+            uint16_t kb = 0, vb = 0;
+            if (tid < g.head_dim) {
+                kb = bf16_bits(k_row);
+                vb = bf16_bits(v_row);
+                a.k_pool_w[tile_at + k_index(P, r_new, tid)] = kb;
+                a.v_pool_w[tile_at + v_index(P, r_new, tid)] = vb;
+            }
+            new_k[tid] = kb;
+            new_v[tid] = vb;
+        }
+    }
+    if (PRE) {
+#pragma unroll
+        for (int u = 0; u < QI; ++u) {
+            const int idx = min(tid + u * THREADS, KK * 64 - 1);
+            const int kk = idx >> 6;
+            const int jj = (idx >> 4) & 3;
+            const int qs = min(idx & 15, rows - 1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                qv[u][e] = pre_out[qs * PS + min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
+        }
     }
 #pragma unroll
     for (int u = 0; u < QI; ++u) {
@@ -402,9 +493,9 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     }
 }
 
-template <int P, int WAVES, bool MQ>
+template <int P, int WAVES, bool MQ, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) void decode_split_kernel(DecodeArgs a) {
-    decode_split_body<P, WAVES, MQ>(a, blockIdx.x, blockIdx.y, blockIdx.z);
+    decode_split_body<P, WAVES, MQ, PRE>(a, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 // Several independent sequences of the same model layer in one launch: grid z is the
@@ -413,7 +504,7 @@ template <int P, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void decode_split_batch_kernel(DecodeBatchArgs b) {
     const DecodeArgs &a = b.seq[blockIdx.z];
     if ((int)blockIdx.x >= a.splits) return;
-    decode_split_body<P, WAVES, false>(a, blockIdx.x, blockIdx.y, 0);
+    decode_split_body<P, WAVES, false, false>(a, blockIdx.x, blockIdx.y, 0);
 }
 
 // ------------------------------------------------------------------------------------
@@ -500,10 +591,11 @@ __global__ __launch_bounds__(256) void decode_merge_batch_kernel(DecodeBatchArgs
     decode_merge_body<MERGE_PER_LANE>(a);
 }
 
-template <int P, int WAVES, bool MQ>
+template <int P, int WAVES, bool MQ, bool PRE>
 static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     constexpr int KK = P / 32;
-    const size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
+    size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
+    if (PRE) stage += ((size_t)2 * 17 * (P + 1) + 3 * P + 22 + 17 * (P + 4)) * sizeof(float);
     const int n_slots = a.n_queries * a.g.gqa;
     const int rows = n_slots < 16 ? n_slots : 16;
     const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
@@ -511,21 +603,24 @@ static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     static bool attr_set = false; // per instantiation
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES, MQ>),
+            reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES, MQ, PRE>),
             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
-    hipLaunchKernelGGL((decode_split_kernel<P, WAVES, MQ>), grid, dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((decode_split_kernel<P, WAVES, MQ, PRE>), grid, dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
 template <int P, int WAVES>
 static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
     // the decode specialisation assumes a single tile of query slots
-    return a.n_queries > 1 || a.g.gqa > 16 ? launch_split_mq<P, WAVES, true>(a, s)
-                                           : launch_split_mq<P, WAVES, false>(a, s);
+    if (a.n_queries > 1 || a.g.gqa > 16) {
+        if (a.pre) return hipErrorInvalidValue; // the caller keeps the fused step to single-tile decode
+        return launch_split_mq<P, WAVES, true, false>(a, s);
+    }
+    return a.pre ? launch_split_mq<P, WAVES, false, true>(a, s) : launch_split_mq<P, WAVES, false, false>(a, s);
 }
 
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {

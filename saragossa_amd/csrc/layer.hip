@@ -135,9 +135,22 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
 // n_queries > 1: chunked prefill over the cache; the last n_queries rows are the new ones
 // and query i attends positions up to len - n_queries + i, each through the layer's
 // sliding window. The matrix-core kernel only.
+// attn_scalar > 0 replaces head_dim under the square root of the score scale
+// (encode_query_attention_scale, src/decode_resident/layers.rs:7-33); pre non-null asks the
+// kernel to norm and rotate q and the new k row itself.
+struct PreKv {
+    const float *rope;
+    const float *q_norm_w;
+    const float *k_norm_w;
+    float eps;
+    int rope_dims;
+    int rope_style;
+};
+
 int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float *out_dev,
                          size_t window_start, const float *k_new = nullptr,
-                         const float *v_new = nullptr, size_t n_queries = 1) {
+                         const float *v_new = nullptr, size_t n_queries = 1,
+                         float attn_scalar = 0.0f, const PreKv *pre = nullptr) {
     int32_t rc = check_window(L, window_start);
     if (rc) return rc;
     const Geom &g = L->g;
@@ -163,13 +176,23 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
         a.scores = L->scores;
         a.len = (long)L->len;
         a.window_start = (long)window_start;
-        a.inv_scale = 1.0f / std::sqrt((float)g.head_dim);
+        a.inv_scale = 1.0f / std::sqrt(attn_scalar > 0.0f ? attn_scalar : (float)g.head_dim);
         a.g = g;
         SKV_HIP(launch_naive(a, s));
         return SKV_OK;
     }
     DecodeArgs a{};
     fill_decode_args(L, q_dev, out_dev, window_start, k_new, v_new, n_queries, decode_target_wgs(), a);
+    if (attn_scalar > 0.0f) a.qscale = (1.0f / std::sqrt(attn_scalar)) * 1.4426950408889634f;
+    if (pre) {
+        a.pre = 1;
+        a.rope = pre->rope;
+        a.q_norm_w = pre->q_norm_w;
+        a.k_norm_w = pre->k_norm_w;
+        a.eps = pre->eps;
+        a.rope_dims = pre->rope ? pre->rope_dims : 0;
+        a.rope_style = pre->rope_style;
+    }
     if (n_queries > 1) {
         // every 16 query slots are a workgroup of their own: split the context only while
         // that leaves compute units idle, and keep the partials in the context's scratch
@@ -588,6 +611,198 @@ int32_t skv_prefill_chunk_host(skv_layer *L, const float *q, const float *k, con
     if (rc) return rc;
     if (e2 != hipSuccess) return fail_hip(e2, "prefill chunk: synchronisation");
     return SKV_OK;
+}
+
+// ---- the step before the cache: per-head RMSNorm + rotation --------------------------
+
+struct skv_rope {
+    skv_ctx *ctx = nullptr;
+    float *table = nullptr; // [max_positions][rope_dims/2][2]
+    size_t max_positions = 0;
+    size_t rope_dims = 0;
+    int style = 0;
+};
+
+int32_t skv_rope_rotations_host(size_t position, size_t rope_dims, size_t frequency_dim, float theta,
+                                float position_scale, float *cos_sin_out) {
+    if (!cos_sin_out) return fail(SKV_ERR_DEVICE, "rope: pointeur nul");
+    if (rope_dims == 0 || rope_dims % 2 != 0)
+        return fail(SKV_ERR_DIMENSION, "RoPE: rope_dims=" + std::to_string(rope_dims) + " doit être pair et non nul");
+    if (!(theta > 0.0f)) return fail(SKV_ERR_DIMENSION, "RoPE: theta doit être > 0");
+    if (frequency_dim == 0) frequency_dim = rope_dims;
+    // rope_rotations (src/decoder/attention_ops.rs:848-887), operation for operation in f32
+    volatile float scaled_position = (float)position * position_scale;
+    for (size_t pair = 0; pair < rope_dims / 2; ++pair) {
+        volatile float exponent = (float)(2 * pair) / (float)frequency_dim;
+        volatile float denom = powf(theta, exponent);
+        volatile float angle = scaled_position / denom;
+        cos_sin_out[2 * pair] = cosf(angle);
+        cos_sin_out[2 * pair + 1] = sinf(angle);
+    }
+    return SKV_OK;
+}
+
+int32_t skv_rope_create(skv_ctx *ctx, size_t max_positions, size_t rope_dims, size_t frequency_dim,
+                        float theta, float position_scale, int32_t style, skv_rope **out) {
+    if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_rope_create: pointeur nul");
+    *out = nullptr;
+    if (max_positions == 0 || max_positions > ((size_t)1 << 30))
+        return fail(SKV_ERR_CONFIG, "RoPE: nombre de positions invalide");
+    if (rope_dims > 512) return fail(SKV_ERR_CONFIG, "RoPE: rope_dims > 512 non supporté");
+    if (style != 0 && style != 1) return fail(SKV_ERR_CONFIG, "RoPE: style inconnu");
+    std::vector<float> host(max_positions * rope_dims);
+    for (size_t p = 0; p < max_positions; ++p) {
+        int32_t rc = skv_rope_rotations_host(p, rope_dims, frequency_dim, theta, position_scale,
+                                             host.data() + p * rope_dims);
+        if (rc) return rc;
+    }
+    SKV_HIP(hipSetDevice(ctx->device));
+    skv_rope *r = new skv_rope();
+    r->ctx = ctx;
+    r->max_positions = max_positions;
+    r->rope_dims = rope_dims;
+    r->style = style;
+    hipError_t e = hipMalloc((void **)&r->table, host.size() * sizeof(float));
+    if (e == hipSuccess)
+        e = hipMemcpy(r->table, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (r->table) (void)hipFree(r->table);
+        delete r;
+        return fail_hip(e, "RoPE: table des rotations");
+    }
+    *out = r;
+    return SKV_OK;
+}
+
+void skv_rope_destroy(skv_rope *rope) {
+    if (!rope) return;
+    (void)hipSetDevice(rope->ctx->device);
+    (void)hipDeviceSynchronize();
+    if (rope->table) (void)hipFree(rope->table);
+    delete rope;
+}
+
+static int32_t check_rope(const skv_rope *rope, size_t position, size_t head_dim) {
+    if (!rope) return SKV_OK;
+    if (rope->rope_dims > head_dim)
+        return fail(SKV_ERR_DIMENSION, "RoPE: rope_dims=" + std::to_string(rope->rope_dims) +
+                                           " > head_dim=" + std::to_string(head_dim));
+    if (position >= rope->max_positions)
+        return fail(SKV_ERR_DIMENSION, "RoPE: position " + std::to_string(position) +
+                                           " hors de la table (" + std::to_string(rope->max_positions) + ")");
+    return SKV_OK;
+}
+
+int32_t skv_rms_norm_rope_decode_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
+                                        size_t position, const float *x_dev, const float *weight_dev,
+                                        size_t heads, size_t head_dim, float eps, float *out_dev) {
+    if (!ctx || !x_dev || !out_dev) return fail(SKV_ERR_DEVICE, "rms_norm_rope: pointeur nul");
+    if (heads == 0 || head_dim == 0 || head_dim > 512 || heads > 65535)
+        return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE heads invalide");
+    int32_t rc = check_rope(rope, position, head_dim);
+    if (rc) return rc;
+    NormRopeArgs a{};
+    a.x = x_dev;
+    a.out = out_dev;
+    a.weight = weight_dev;
+    a.rope = rope ? rope->table + position * rope->rope_dims : nullptr;
+    a.heads = (int)heads;
+    a.head_dim = (int)head_dim;
+    a.rope_dims = rope ? (int)rope->rope_dims : 0;
+    a.rope_style = rope ? rope->style : 0;
+    a.eps = eps;
+    SKV_HIP(launch_norm_rope(a, as_stream(stream)));
+    return SKV_OK;
+}
+
+int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float *weight, size_t heads,
+                                      size_t head_dim, size_t rope_dims, size_t frequency_dim,
+                                      size_t position, float eps, float theta, float position_scale,
+                                      int32_t style, float *out) {
+    if (!ctx || !x || !out) return fail(SKV_ERR_DEVICE, "rms_norm_rope: pointeur nul");
+    if (heads == 0 || head_dim == 0 || head_dim > 512 || heads > 65535)
+        return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE heads invalide");
+    if (rope_dims == 0 || rope_dims > head_dim || rope_dims % 2 != 0)
+        return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE: rope_dims invalide");
+    if (style != 0 && style != 1) return fail(SKV_ERR_CONFIG, "RoPE: style inconnu");
+    std::vector<float> cs(rope_dims);
+    int32_t rc = skv_rope_rotations_host(position, rope_dims, frequency_dim, theta, position_scale, cs.data());
+    if (rc) return rc;
+    SKV_HIP(hipSetDevice(ctx->device));
+    const size_t n = heads * head_dim;
+    float *buf = nullptr;
+    SKV_HIP(hipMalloc((void **)&buf, (2 * n + head_dim + rope_dims) * sizeof(float)));
+    float *xd = buf, *od = buf + n, *wd = buf + 2 * n, *rd = wd + head_dim;
+    hipStream_t s = ctx->stream;
+    hipError_t e = hipMemcpyAsync(xd, x, n * sizeof(float), hipMemcpyHostToDevice, s);
+    if (e == hipSuccess && weight) e = hipMemcpyAsync(wd, weight, head_dim * sizeof(float), hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(rd, cs.data(), rope_dims * sizeof(float), hipMemcpyHostToDevice, s);
+    NormRopeArgs a{};
+    a.x = xd;
+    a.out = od;
+    a.weight = weight ? wd : nullptr;
+    a.rope = rd;
+    a.heads = (int)heads;
+    a.head_dim = (int)head_dim;
+    a.rope_dims = (int)rope_dims;
+    a.rope_style = style;
+    a.eps = eps;
+    if (e == hipSuccess) e = launch_norm_rope(a, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(out, od, n * sizeof(float), hipMemcpyDeviceToHost, s);
+    hipError_t e2 = hipStreamSynchronize(s);
+    (void)hipFree(buf);
+    if (e != hipSuccess) return fail_hip(e, "rms_norm_rope");
+    if (e2 != hipSuccess) return fail_hip(e2, "rms_norm_rope: synchronisation");
+    return SKV_OK;
+}
+
+int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_rope *rope,
+                                     size_t position, const void *q_dev, size_t q_off,
+                                     const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
+                                     const float *q_norm_w, const float *k_norm_w, float eps,
+                                     float attn_scalar, float *out_dev) {
+    if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step_prekv: pointeur nul");
+    if ((q_off | k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "decode_step_prekv: offset non aligné f32");
+    if (!std::isfinite(attn_scalar) || attn_scalar <= 0.0f)
+        return fail(SKV_ERR_CONFIG, "scalaire d'attention résident invalide: " + std::to_string(attn_scalar));
+    int32_t rc = check_rope(rope, position, (size_t)L->g.head_dim);
+    if (rc) return rc;
+    if (L->len >= L->capacity)
+        return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
+                                           std::to_string(L->capacity) + " atteinte (overflow)");
+    const float *q = reinterpret_cast<const float *>((const char *)q_dev + q_off);
+    const float *k = reinterpret_cast<const float *>((const char *)k_dev + k_off);
+    const float *v = reinterpret_cast<const float *>((const char *)v_dev + v_off);
+    hipStream_t s = as_stream(stream);
+    static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
+    if (!fused || !uses_flash(L) || L->g.gqa > 16) {
+        // the same step as separate launches: norm + rotation of q and k, append, attention
+        rc = skv_rms_norm_rope_decode_device(L->ctx, stream, rope, position, q, q_norm_w,
+                                             (size_t)L->g.q_heads, (size_t)L->g.head_dim, eps, L->q_stage);
+        if (rc) return rc;
+        rc = skv_rms_norm_rope_decode_device(L->ctx, stream, rope, position, k, k_norm_w,
+                                             (size_t)L->g.kv_heads, (size_t)L->g.head_dim, eps, L->kv_stage);
+        if (rc) return rc;
+        rc = encode_append(L, s, L->kv_stage, v, 1);
+        if (rc) return rc;
+        return encode_attention(L, s, L->q_stage, out_dev, skv_window_start(L->len - 1, L->window),
+                                nullptr, nullptr, 1, attn_scalar);
+    }
+    PreKv pre{};
+    pre.rope = rope ? rope->table + position * rope->rope_dims : nullptr;
+    pre.q_norm_w = q_norm_w;
+    pre.k_norm_w = k_norm_w;
+    pre.eps = eps;
+    pre.rope_dims = rope ? (int)rope->rope_dims : 0;
+    pre.rope_style = rope ? rope->style : 0;
+    L->len += 1;
+    if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
+        L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
+    rc = encode_attention(L, s, q, out_dev, skv_window_start(L->len - 1, L->window), k, v, 1,
+                          attn_scalar, &pre);
+    if (rc) L->len -= 1;
+    return rc;
 }
 
 int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_stream stream,

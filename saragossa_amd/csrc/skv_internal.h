@@ -109,8 +109,94 @@ struct DecodeArgs {
     uint16_t *k_pool_w;
     uint16_t *v_pool_w;
     int new_slot;     // slot that receives the row
+    // fused pre-KV step (pre != 0): q and the appended k row arrive raw and get the per-head
+    // RMSNorm (weights null = none) and the rotation of this position before they are used
+    int pre;
+    int rope_dims;          // rotated leading dims of each head (even, <= head_dim; 0 = none)
+    int rope_style;         // 0 = halves (i, i + rope_dims/2), 1 = interleaved (2i, 2i+1)
+    float eps;
+    const float *rope;      // [rope_dims/2][2]: (cos, sin) of this position
+    const float *q_norm_w;  // [head_dim]
+    const float *k_norm_w;  // [head_dim]
     Geom g;
 };
+static_assert(sizeof(DecodeArgs) <= 256, "sixteen of them must fit the kernel argument block");
+
+// Standalone per-head RMSNorm + rotation of one row (the same arithmetic as the fused step).
+struct NormRopeArgs {
+    const float *x;      // [heads][head_dim]
+    float *out;          // [heads][head_dim]
+    const float *weight; // [head_dim] or null
+    const float *rope;   // [rope_dims/2][2] or null
+    int heads, head_dim, rope_dims, rope_style;
+    float eps;
+};
+hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s);
+
+#ifdef __HIPCC__
+// The arithmetic of rms_norm_rope_heads_at (src/decoder/attention_ops.rs:682-777), operation
+// for operation and without contraction, so that the device row equals the CPU row bit for
+// bit when the (cos, sin) table comes from the host's libm.
+// (The contraction pragma matters: the __f*_rn intrinsics are plain operators here and
+// would be fused into FMAs otherwise.)
+__device__ __forceinline__ float head_inv_rms(const float *row, int head_dim, float eps) {
+#pragma clang fp contract(off)
+    float sum = 0.0f;
+    for (int c = 0; c < head_dim; ++c) {
+        const float sq = row[c] * row[c];
+        sum = sum + sq;
+    }
+    const float mean_square = sum / (float)head_dim;
+    return 1.0f / sqrtf(mean_square + eps);
+}
+// The same from the squares, already taken (x * x, rounded) and padded with zeros to a
+// multiple of 16 entries at a 16-byte aligned address: the adds stay in index order, the
+// loads come sixteen values at a time.
+__device__ __forceinline__ float head_inv_rms_sq(const float *sq, int padded, int head_dim, float eps) {
+#pragma clang fp contract(off)
+    typedef __attribute__((ext_vector_type(4))) float f4;
+    const f4 *p = reinterpret_cast<const f4 *>(sq);
+    float sum = 0.0f;
+    for (int c = 0; c < padded / 4; c += 4) {
+        const f4 v0 = p[c], v1 = p[c + 1], v2 = p[c + 2], v3 = p[c + 3];
+        sum = sum + v0.x; sum = sum + v0.y; sum = sum + v0.z; sum = sum + v0.w;
+        sum = sum + v1.x; sum = sum + v1.y; sum = sum + v1.z; sum = sum + v1.w;
+        sum = sum + v2.x; sum = sum + v2.y; sum = sum + v2.z; sum = sum + v2.w;
+        sum = sum + v3.x; sum = sum + v3.y; sum = sum + v3.z; sum = sum + v3.w;
+    }
+    const float mean_square = sum / (float)head_dim;
+    return 1.0f / sqrtf(mean_square + eps);
+}
+// Element c of the head after norm (inv, w; w null = 1) and rotation (rope null = none).
+__device__ __forceinline__ float norm_rope_elem(const float *row, int c, float inv, const float *w,
+                                                const float *rope, int rope_dims, int style) {
+#pragma clang fp contract(off)
+    auto normed = [&](int i) {
+#pragma clang fp contract(off)
+        const float scaled = row[i] * inv;
+        return w ? scaled * w[i] : scaled;
+    };
+    if (!rope || c >= rope_dims) return normed(c);
+    const int pairs = rope_dims >> 1;
+    int pair, i0, i1;
+    bool is_first;
+    if (style == 1) {
+        pair = c >> 1;
+        i0 = 2 * pair;
+        i1 = i0 + 1;
+        is_first = (c & 1) == 0;
+    } else {
+        is_first = c < pairs;
+        pair = is_first ? c : c - pairs;
+        i0 = pair;
+        i1 = pair + pairs;
+    }
+    const float cs = rope[2 * pair], sn = rope[2 * pair + 1];
+    const float first = normed(i0), second = normed(i1);
+    const float fc = first * cs, ss = second * sn, fs = first * sn, sc = second * cs;
+    return is_first ? fc - ss : fs + sc;
+}
+#endif
 
 // One decode step of the same model layer for several independent sequences.
 constexpr int SKV_MAX_BATCH = 16;

@@ -56,10 +56,59 @@ class DecodeResidentState:
                                            int(sampled), C.byref(h)))
         return FullAttentionState(self, h)
 
+    def rms_norm_rope_decode(self, x, weight, heads, head_dim, rope_dims, position, eps, theta,
+                             position_scale=1.0, frequency_dim=0, style=0) -> np.ndarray:
+        """DecodeResidentState::rms_norm_rope_decode (src/decode_resident/tests.rs:1168-1172);
+        weight None = rotation only."""
+        xa = _f32(x).reshape(-1)
+        out = np.empty_like(xa)
+        w = None if weight is None else _f32(weight).reshape(-1)
+        if xa.size != heads * head_dim or (w is not None and w.size != head_dim):
+            from ._lib import DimensionError
+            raise DimensionError("RMSNorm/RoPE heads invalide")
+        check(self._l.skv_rms_norm_rope_decode_host(self._h, _p(xa), None if w is None else _p(w),
+                                                    heads, head_dim, rope_dims, frequency_dim,
+                                                    position, eps, theta, position_scale, style,
+                                                    _p(out)))
+        return out
+
+    def rope_table(self, max_positions, rope_dims, theta, position_scale=1.0, frequency_dim=0,
+                   style=0) -> "RopeTable":
+        return RopeTable(self, max_positions, rope_dims, theta, position_scale, frequency_dim, style)
+
     def full_attention_bf16(self, capacity, q_heads, kv_heads, head_dim, window=0):
         """full_attention_bf16_for_test (attention.rs:47-54)."""
         return self.full_attention_with_element(capacity, q_heads, kv_heads, head_dim,
                                                 DTYPE_BF16, window)
+
+
+def rope_rotations(position, rope_dims, theta, position_scale=1.0, frequency_dim=0) -> np.ndarray:
+    """rope_rotations (src/decoder/attention_ops.rs:848-887) on the host: [rope_dims/2, 2] of
+    (cos, sin)."""
+    out = np.empty(rope_dims, np.float32)
+    check(lib().skv_rope_rotations_host(position, rope_dims, frequency_dim, theta, position_scale,
+                                        _p(out)))
+    return out.reshape(-1, 2)
+
+
+class RopeTable:
+    """Device table of the rotations of positions 0..max_positions-1 (skv_rope_create)."""
+
+    def __init__(self, ctx, max_positions, rope_dims, theta, position_scale=1.0, frequency_dim=0,
+                 style=0):
+        self._ctx, self._l = ctx, ctx._l
+        h = C.c_void_p()
+        check(self._l.skv_rope_create(ctx._h, max_positions, rope_dims, frequency_dim, theta,
+                                      position_scale, style, C.byref(h)))
+        self._h = h
+
+    def close(self) -> None:
+        if getattr(self, "_h", None):
+            self._l.skv_rope_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
 
 
 class FullAttentionState:
@@ -171,6 +220,14 @@ class FullAttentionState:
     def encode_decode_step(self, stream, k_ptr, k_off, v_ptr, v_off, q_ptr, out_ptr) -> None:
         check(self._l.skv_decode_step_device(self._h, stream, k_ptr, k_off, v_ptr, v_off, q_ptr,
                                              out_ptr))
+
+    def encode_decode_step_prekv(self, stream, rope, position, q_ptr, q_off, k_ptr, k_off, v_ptr,
+                                 v_off, q_norm_ptr, k_norm_ptr, eps, attn_scalar, out_ptr) -> None:
+        """The q/k norms, rotation, query scale, append and attention of
+        encode_resident_full_layer (src/decode_resident/layers.rs:214-288) in one call."""
+        check(self._l.skv_decode_step_prekv_device(
+            self._h, stream, None if rope is None else rope._h, position, q_ptr, q_off, k_ptr,
+            k_off, v_ptr, v_off, q_norm_ptr, k_norm_ptr, eps, attn_scalar, out_ptr))
 
     def encode_gather(self, stream, first, n, k_dst_ptr, v_dst_ptr) -> None:
         check(self._l.skv_gather_device(self._h, stream, first, n, k_dst_ptr, v_dst_ptr))
