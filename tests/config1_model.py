@@ -101,6 +101,54 @@ class OracleKv:
         return self.caches[li].keys(), self.caches[li].values()
 
 
+def norm_rope_cpu(x, heads, cfg, position):
+    """rms_norm_rope_heads_at on the CPU oracle (unit norm weights), rows at position.."""
+    ones = np.ones(cfg.head_dim, np.float32)
+    return oracle.rms_norm_rope_heads_at(x.cpu().numpy(), heads, cfg.head_dim, cfg.head_dim, ones,
+                                         cfg.eps, cfg.theta, position)
+
+
+class HipKvPre(HipKv):
+    """As HipKv, but a decode token hands the raw q and k projections to the library, which
+    applies the q/k norms and the rotation itself (the fused step before the cache). Prefill
+    chunks take their norm + rotation from the CPU oracle, as the other arm does."""
+    raw_qk = True
+
+    def __init__(self, cfg, capacity, state, seed=0):
+        super().__init__(cfg, capacity, state, seed)
+        self.cfg = cfg
+        self.rope = state.rope_table(capacity, cfg.head_dim, cfg.theta)
+        self.ones = torch.ones(cfg.head_dim, device="cuda")
+
+    def attend_raw(self, li, q_raw, k_raw, v, position):
+        cfg = self.cfg
+        if q_raw.shape[0] == 1:
+            out = torch.empty_like(q_raw)
+            self.layers[li].encode_decode_step_prekv(
+                self.stream, self.rope, position, q_raw.data_ptr(), 0, k_raw.data_ptr(), 0,
+                v.data_ptr(), 0, self.ones.data_ptr(), self.ones.data_ptr(), cfg.eps,
+                float(cfg.head_dim), out.data_ptr())
+            return out
+        q = torch.from_numpy(norm_rope_cpu(q_raw, cfg.q_heads, cfg, position)).cuda()
+        k = torch.from_numpy(norm_rope_cpu(k_raw, cfg.kv_heads, cfg, position)).cuda()
+        return self.attend(li, q, k, v)
+
+
+class OracleKvPre(OracleKv):
+    """The CPU path end to end for the attention block: rms_norm_rope_heads_at, append,
+    cached_attention_one."""
+    raw_qk = True
+
+    def __init__(self, cfg, capacity=None, state=None, seed=0):
+        super().__init__(cfg, capacity, state, seed)
+        self.cfg = cfg
+
+    def attend_raw(self, li, q_raw, k_raw, v, position):
+        q = torch.from_numpy(norm_rope_cpu(q_raw, self.cfg.q_heads, self.cfg, position)).cuda()
+        k = torch.from_numpy(norm_rope_cpu(k_raw, self.cfg.kv_heads, self.cfg, position)).cuda()
+        return self.attend(li, q, k, v)
+
+
 def forward(cfg, w, kv, tokens, position):
     """Runs `tokens` (a chunk, or one token) at positions position.. and returns the last
     row's logits."""
@@ -109,10 +157,14 @@ def forward(cfg, w, kv, tokens, position):
     x = w.embed[ids]
     for li, lw in enumerate(w.layers):
         h = rms_norm(x, w.ones_h, cfg.eps)
-        q = norm_rope(h @ lw["wq"].T, cfg.q_heads, cfg.head_dim, w.ones_d, cfg.eps, cfg.theta, pos)
-        k = norm_rope(h @ lw["wk"].T, cfg.kv_heads, cfg.head_dim, w.ones_d, cfg.eps, cfg.theta, pos)
         v = (h @ lw["wv"].T).contiguous()
-        ctx = kv.attend(li, q.contiguous(), k.contiguous(), v)
+        if getattr(kv, "raw_qk", False):
+            ctx = kv.attend_raw(li, (h @ lw["wq"].T).contiguous(), (h @ lw["wk"].T).contiguous(), v,
+                                position)
+        else:
+            q = norm_rope(h @ lw["wq"].T, cfg.q_heads, cfg.head_dim, w.ones_d, cfg.eps, cfg.theta, pos)
+            k = norm_rope(h @ lw["wk"].T, cfg.kv_heads, cfg.head_dim, w.ones_d, cfg.eps, cfg.theta, pos)
+            ctx = kv.attend(li, q.contiguous(), k.contiguous(), v)
         x = x + ctx @ lw["wo"].T
         h2 = rms_norm(x, w.ones_h, cfg.eps)
         x = x + (torch.nn.functional.silu(h2 @ lw["wg"].T) * (h2 @ lw["wu"].T)) @ lw["wd"].T

@@ -12,22 +12,26 @@ import pytest
 pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
-from config1_model import Config, HipKv, OracleKv, Weights, greedy  # noqa: E402
+from config1_model import Config, HipKv, HipKvPre, OracleKv, OracleKvPre, Weights, greedy  # noqa: E402
 
 FULL = os.environ.get("SKV_FULL_CONFIG1") == "1"
 
 
 @pytest.mark.timeout(3000 if FULL else 300)
-def test_config1_greedy_ids_match_oracle(state):
+@pytest.mark.parametrize("hip_cls,ora_cls", [(HipKv, OracleKv), (HipKvPre, OracleKvPre)],
+                         ids=["kv-path", "fused-pre-kv"])
+def test_config1_greedy_ids_match_oracle(state, hip_cls, ora_cls):
+    """ids "fused-pre-kv": decode tokens additionally run the q/k norms and the rotation
+    inside the library's fused step (device) against rms_norm_rope_heads_at (CPU)."""
     cfg = Config() if FULL else Config(layers=4)
     n_prompt, n_new, chunk = (2048, 256, 512) if FULL else (256, 48, 96)
     w = Weights(cfg, seed=1)
     prompt = [int(t) for t in np.random.default_rng(1).integers(0, cfg.vocab, size=n_prompt)]
     cap = n_prompt + n_new
     with torch.no_grad():
-        hip = HipKv(cfg, cap, state)
+        hip = hip_cls(cfg, cap, state)
         ids_hip, margins, logits_hip = greedy(cfg, w, hip, prompt, n_new, chunk)
-        ora = OracleKv(cfg)
+        ora = ora_cls(cfg)
         ids_ora, _, logits_ora = greedy(cfg, w, ora, prompt, n_new, chunk)
     print(f"config1 {'full' if FULL else 'reduced'}: min top-1/top-2 margin {min(margins):.3e}, "
           f"max |logit diff| {max(float(np.abs(a - b).max()) for a, b in zip(logits_hip, logits_ora)):.3e}")
