@@ -213,6 +213,23 @@ int32_t skv_decode_step_prekv_device(skv_layer *layer, skv_stream stream, const 
                                      const float *q_norm_w, const float *k_norm_w, float eps,
                                      float attn_scalar, float *out_dev);
 
+/* The same step for a layer with an output gate (attn_output_gate, Qwen3.5/3.6 full-attention
+ * layers): qg_dev + qg_off is the gated q projection, per head head_dim query values then
+ * head_dim gate values (split_q_gate_f32, src/decode_resident/kernels.rs:931-946;
+ * split_attention_gate, src/decoder/attention_ops.rs:486-520), read in place; the context
+ * leaves the kernel already multiplied by sigmoid(gate) (attn_gate_f32, kernels.rs:949-959;
+ * attention_ops.rs:217-219, 522-524), ready for the o projection. */
+int32_t skv_decode_step_gated_device(skv_layer *layer, skv_stream stream, const skv_rope *rope,
+                                     size_t position, const void *qg_dev, size_t qg_off,
+                                     const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
+                                     const float *q_norm_w, const float *k_norm_w, float eps,
+                                     float attn_scalar, float *out_dev);
+/* encode_attn_gate (attn_gate_f32, src/decode_resident/kernels.rs:949-959) on its own:
+ * out[h][c] = ctx[h][c] * sigmoid(gate[h * gate_head_stride + c]); stride 0 = head_dim;
+ * out may be ctx. */
+int32_t skv_attn_gate_device(skv_ctx *ctx, skv_stream stream, const float *ctx_dev, const float *gate_dev,
+                             size_t gate_head_stride, size_t heads, size_t head_dim, float *out_dev);
+
 /* One decode step of the SAME model layer for n_seq independent sequences (each its own
  * handle, block table and length): for sequence i, append k_dev[i]/v_dev[i] (kv_dim f32
  * each) then attention of q_dev[i] into out_dev[i], all in one pair of launches. The

@@ -125,6 +125,12 @@ def lib():
                                                C.c_size_t, C.c_int, C.c_void_p]
         l.skvo_sdpa_2pass_blocks.restype = C.c_size_t
         l.skvo_sdpa_2pass_blocks.argtypes = [C.c_size_t]
+        l.skvo_split_attention_gate.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t,
+                                                C.c_size_t, C.c_void_p, C.c_void_p]
+        l.skvo_attention_gate.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        l.skvo_attention_gate.restype = None
+        l.skvo_sigmoid.restype = C.c_float
+        l.skvo_sigmoid.argtypes = [C.c_float]
         l.skvo_window_start.restype = C.c_size_t
         l.skvo_window_start.argtypes = [C.c_size_t, C.c_size_t]
         l.skvo_resident_capacity.restype = C.c_int
@@ -319,6 +325,26 @@ def apply_rope_heads_at(x, heads, head_dim, rope_dims, theta, position_offset, s
     _check(lib().skvo_apply_rope_heads_at(_ptr(xa), xa.shape[0], heads, head_dim, rope_dims, theta,
                                           position_scale, frequency_dim or rope_dims,
                                           position_offset, style, _ptr(out)), "RoPE")
+    return out
+
+
+def split_attention_gate(q_projection, heads, head_dim):
+    """split_attention_gate (src/decoder/attention_ops.rs:486-520): ([rows, q_dim] q, gate)."""
+    qp = np.atleast_2d(_f32(q_projection))
+    q = np.empty((qp.shape[0], heads * head_dim), np.float32)
+    gate = np.empty_like(q)
+    _check(lib().skvo_split_attention_gate(_ptr(qp), qp.shape[0], qp.shape[1], heads, head_dim,
+                                           _ptr(q), _ptr(gate)), "q_proj gated")
+    return q, gate
+
+
+def attention_gate(context, gate):
+    """context * sigmoid(gate) (src/decoder/attention_ops.rs:217-219, 522-524)."""
+    c, g = _f32(context), _f32(gate)
+    if c.shape != g.shape:
+        raise OracleError(ERR_DIMENSION, "gate shape")
+    out = np.empty_like(c)
+    lib().skvo_attention_gate(_ptr(c), _ptr(g), c.size, _ptr(out))
     return out
 
 

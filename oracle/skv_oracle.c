@@ -23,6 +23,8 @@
  *   skvo_causal_attention                      equality with the cached path row by row, fp64 bound
  *   skvo_cached_attention_prefill_rows         definitionally append + attention per row
  *   skvo_rms_norm_rope_heads_at / apply_rope   MLX-captured constants (src/decoder/tests.rs:998-1113)
+ *   skvo_split_attention_gate, skvo_attention_gate   index identity against a reshape; sigmoid(0) = 1/2,
+ *                                             sigmoid(x) + sigmoid(-x) = 1, fp64 formula to one ulp
  *   skvo_sdpa_2pass_blocks, skvo_window_start  integer closed forms from the reference's comments
  * The last-ulp value of the float functions on large random inputs is pinned
  * only by the same-libm/no-contraction argument above: parity unpinned beyond
@@ -553,6 +555,34 @@ int skvo_apply_rope_heads_at(const float *x, size_t seq, size_t heads, size_t he
     free(cosv);
     free(sinv);
     return SKVO_OK;
+}
+
+/* ---- output gate --------------------------------------------------------- */
+
+/* split_attention_gate (src/decoder/attention_ops.rs:486-520): the gated q projection
+ * holds, per head, head_dim query values then head_dim gate values. */
+int skvo_split_attention_gate(const float *q_projection, size_t rows, size_t cols, size_t heads,
+                              size_t head_dim, float *q, float *gate) {
+    size_t q_dim = heads * head_dim;
+    if (heads == 0 || head_dim == 0 || cols != 2 * q_dim) return SKVO_ERR_DIMENSION;
+    for (size_t row = 0; row < rows; ++row) {
+        const float *source = q_projection + row * cols;
+        for (size_t head = 0; head < heads; ++head) {
+            size_t start = head * 2 * q_dim / heads;
+            memcpy(q + row * q_dim + head * head_dim, source + start, head_dim * sizeof(float));
+            memcpy(gate + row * q_dim + head * head_dim, source + start + head_dim,
+                   head_dim * sizeof(float));
+        }
+    }
+    return SKVO_OK;
+}
+
+/* sigmoid_scalar (src/decoder/attention_ops.rs:522-524). */
+float skvo_sigmoid(float value) { return 1.0f / (1.0f + expf(-value)); }
+
+/* context.mul_elementwise(gate.map(sigmoid_scalar)) (src/decoder/attention_ops.rs:217-219). */
+void skvo_attention_gate(const float *context, const float *gate, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) out[i] = context[i] * skvo_sigmoid(gate[i]);
 }
 
 /* ---- integer policy helpers --------------------------------------------- */

@@ -93,6 +93,9 @@ SIGNATURES = {
                                              C.c_float, C.c_float, _i32, _vp]),
     "skv_decode_step_prekv_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp,
                                             C.c_float, C.c_float, _vp]),
+    "skv_decode_step_gated_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp,
+                                            C.c_float, C.c_float, _vp]),
+    "skv_attn_gate_device": (_i32, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "skv_decode_step_batch_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_decode_step_layers_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_read_rows": (_i32, [_vp, _sz, _sz, _vp, _vp]),

@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(NormRopeArgs a) {
     __shared__ float inv_s;
     const int head = blockIdx.x;
     const int tid = threadIdx.x;
-    const float *x = a.x + (long)head * a.head_dim;
+    const float *x = a.x + (long)head * (a.x_head_stride > 0 ? a.x_head_stride : a.head_dim);
     for (int c = tid; c < a.head_dim; c += 256) {
         row[c] = x[c];
         w[c] = a.weight ? a.weight[c] : 1.0f;
@@ -214,6 +214,22 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(NormRopeArgs a) {
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s) {
     if (a.heads <= 0 || a.head_dim <= 0 || a.head_dim > 512) return hipErrorInvalidValue;
     hipLaunchKernelGGL(norm_rope_kernel, dim3((unsigned)a.heads), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+// out = ctx * sigmoid(gate) (attn_gate_f32, src/decode_resident/kernels.rs:949-959); the
+// gate may sit interleaved with q in the gated q projection (gate_head_stride = 2 * head_dim).
+__global__ __launch_bounds__(256) void gate_kernel(GateArgs a) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.heads * a.head_dim) return;
+    const int h = i / a.head_dim, c = i - h * a.head_dim;
+    a.out[i] = a.ctx[i] * sigmoid_gate(a.gate[(long)h * a.gate_head_stride + c]);
+}
+
+hipError_t launch_gate(const GateArgs &a, hipStream_t s) {
+    const int n = a.heads * a.head_dim;
+    if (n <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gate_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

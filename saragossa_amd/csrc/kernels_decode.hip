@@ -90,6 +90,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     const int n = lane & 15; // key row inside the tile (A operand) / query slot (B, D)
     const int j = lane >> 4;
     const int tile = MQ ? tile_z : 0;
+    const int q_stride = (!MQ && a.q_head_stride > 0) ? a.q_head_stride : g.head_dim;
     const int G = g.gqa;
     const int C = MQ ? a.n_queries : 1;
     const int n_slots = C * G;
@@ -155,7 +156,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         for (int u = 0; u < PRE_U; ++u) {
             const int e = tid + u * THREADS;
             const int r = e / P, c = e % P;
-            pre_q[u] = (r < rows && c < g.head_dim) ? a.q[(long)(kvh * G + r) * g.head_dim + c] : 0.0f;
+            pre_q[u] = (r < rows && c < g.head_dim) ? a.q[(long)(kvh * G + r) * q_stride + c] : 0.0f;
         }
         if (tid < g.head_dim) {
             if (a.q_norm_w) pre_w0 = a.q_norm_w[tid];
@@ -185,8 +186,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         const int kk = idx >> 6;
         const int jj = (idx >> 4) & 3;
         const int qs = min(tile * 16 + (idx & 15), n_slots - 1);
-        const float *qrow = a.q + (MQ ? ((long)(qs / G) * g.q_heads + kvh * G + qs % G)
-                                      : (long)(kvh * G + qs)) * g.head_dim;
+        const float *qrow = MQ ? a.q + ((long)(qs / G) * g.q_heads + kvh * G + qs % G) * g.head_dim
+                               : a.q + (long)(kvh * G + qs) * q_stride;
 #pragma unroll
         for (int e = 0; e < 8; ++e) qv[u][e] = qrow[min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
     }
@@ -471,6 +472,12 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         float *dst;
         if (a.splits == 1) {
             acc *= 1.0f / lsum;
+            if (!MQ && a.gate) {
+                const float *gp = a.gate + (long)(kvh * G + slot) * q_stride + c4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (c4 + i < g.head_dim) acc[i] *= sigmoid_gate(gp[i]);
+            }
             dst = a.out + (MQ ? ((long)(slot / G) * g.q_heads + kvh * G + slot % G)
                               : (long)(kvh * G + slot)) * g.head_dim + c4;
         } else {
@@ -574,7 +581,10 @@ __device__ __forceinline__ void decode_merge_body(const DecodeArgs &a) {
             t += acc_x[i][c];
             l += red_l[i];
         }
-        a.out[h * g.head_dim + col] = t / l;
+        float r = t / l;
+        if (a.gate && a.n_queries == 1)
+            r *= sigmoid_gate(a.gate[h * (a.q_head_stride > 0 ? a.q_head_stride : g.head_dim) + col]);
+        a.out[h * g.head_dim + col] = r;
     }
 }
 

@@ -145,6 +145,8 @@ struct PreKv {
     float eps;
     int rope_dims;
     int rope_style;
+    const float *gate;  // multiplied into the context through a sigmoid (null = none)
+    int q_head_stride;  // elements between the heads of q and of gate (0 = head_dim)
 };
 
 int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float *out_dev,
@@ -192,6 +194,8 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
         a.eps = pre->eps;
         a.rope_dims = pre->rope ? pre->rope_dims : 0;
         a.rope_style = pre->rope_style;
+        a.gate = pre->gate;
+        a.q_head_stride = pre->q_head_stride;
     }
     if (n_queries > 1) {
         // every 16 query slots are a workgroup of their own: split the context only while
@@ -756,14 +760,10 @@ int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float 
     return SKV_OK;
 }
 
-int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_rope *rope,
-                                     size_t position, const void *q_dev, size_t q_off,
-                                     const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
-                                     const float *q_norm_w, const float *k_norm_w, float eps,
-                                     float attn_scalar, float *out_dev) {
-    if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
-        return fail(SKV_ERR_DEVICE, "decode_step_prekv: pointeur nul");
-    if ((q_off | k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "decode_step_prekv: offset non aligné f32");
+static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope, size_t position,
+                          const float *q, size_t q_head_stride, const float *gate, const float *k,
+                          const float *v, const float *q_norm_w, const float *k_norm_w, float eps,
+                          float attn_scalar, float *out_dev) {
     if (!std::isfinite(attn_scalar) || attn_scalar <= 0.0f)
         return fail(SKV_ERR_CONFIG, "scalaire d'attention résident invalide: " + std::to_string(attn_scalar));
     int32_t rc = check_rope(rope, position, (size_t)L->g.head_dim);
@@ -771,23 +771,42 @@ int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_
     if (L->len >= L->capacity)
         return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
                                            std::to_string(L->capacity) + " atteinte (overflow)");
-    const float *q = reinterpret_cast<const float *>((const char *)q_dev + q_off);
-    const float *k = reinterpret_cast<const float *>((const char *)k_dev + k_off);
-    const float *v = reinterpret_cast<const float *>((const char *)v_dev + v_off);
     hipStream_t s = as_stream(stream);
     static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
     if (!fused || !uses_flash(L) || L->g.gqa > 16) {
-        // the same step as separate launches: norm + rotation of q and k, append, attention
-        rc = skv_rms_norm_rope_decode_device(L->ctx, stream, rope, position, q, q_norm_w,
-                                             (size_t)L->g.q_heads, (size_t)L->g.head_dim, eps, L->q_stage);
-        if (rc) return rc;
-        rc = skv_rms_norm_rope_decode_device(L->ctx, stream, rope, position, k, k_norm_w,
-                                             (size_t)L->g.kv_heads, (size_t)L->g.head_dim, eps, L->kv_stage);
-        if (rc) return rc;
+        // the same step as separate launches: norm + rotation of q and k, append, attention, gate
+        NormRopeArgs n{};
+        n.x = q;
+        n.out = L->q_stage;
+        n.weight = q_norm_w;
+        n.rope = rope ? rope->table + position * rope->rope_dims : nullptr;
+        n.heads = L->g.q_heads;
+        n.head_dim = L->g.head_dim;
+        n.rope_dims = rope ? (int)rope->rope_dims : 0;
+        n.rope_style = rope ? rope->style : 0;
+        n.eps = eps;
+        n.x_head_stride = (int)q_head_stride;
+        SKV_HIP(launch_norm_rope(n, s));
+        n.x = k;
+        n.out = L->kv_stage;
+        n.weight = k_norm_w;
+        n.heads = L->g.kv_heads;
+        n.x_head_stride = 0;
+        SKV_HIP(launch_norm_rope(n, s));
         rc = encode_append(L, s, L->kv_stage, v, 1);
         if (rc) return rc;
-        return encode_attention(L, s, L->q_stage, out_dev, skv_window_start(L->len - 1, L->window),
-                                nullptr, nullptr, 1, attn_scalar);
+        rc = encode_attention(L, s, L->q_stage, out_dev, skv_window_start(L->len - 1, L->window),
+                              nullptr, nullptr, 1, attn_scalar);
+        if (rc || !gate) return rc;
+        GateArgs ga{};
+        ga.ctx = out_dev;
+        ga.gate = gate;
+        ga.out = out_dev;
+        ga.heads = L->g.q_heads;
+        ga.head_dim = L->g.head_dim;
+        ga.gate_head_stride = q_head_stride ? (int)q_head_stride : L->g.head_dim;
+        SKV_HIP(launch_gate(ga, s));
+        return SKV_OK;
     }
     PreKv pre{};
     pre.rope = rope ? rope->table + position * rope->rope_dims : nullptr;
@@ -796,6 +815,8 @@ int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_
     pre.eps = eps;
     pre.rope_dims = rope ? (int)rope->rope_dims : 0;
     pre.rope_style = rope ? rope->style : 0;
+    pre.gate = gate;
+    pre.q_head_stride = (int)q_head_stride;
     L->len += 1;
     if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
         L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
@@ -803,6 +824,57 @@ int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_
                           attn_scalar, &pre);
     if (rc) L->len -= 1;
     return rc;
+}
+
+int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_rope *rope,
+                                     size_t position, const void *q_dev, size_t q_off,
+                                     const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
+                                     const float *q_norm_w, const float *k_norm_w, float eps,
+                                     float attn_scalar, float *out_dev) {
+    if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step_prekv: pointeur nul");
+    if ((q_off | k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "decode_step_prekv: offset non aligné f32");
+    return prekv_step(L, stream, rope, position,
+                      reinterpret_cast<const float *>((const char *)q_dev + q_off), 0, nullptr,
+                      reinterpret_cast<const float *>((const char *)k_dev + k_off),
+                      reinterpret_cast<const float *>((const char *)v_dev + v_off), q_norm_w,
+                      k_norm_w, eps, attn_scalar, out_dev);
+}
+
+int32_t skv_decode_step_gated_device(skv_layer *L, skv_stream stream, const skv_rope *rope,
+                                     size_t position, const void *qg_dev, size_t qg_off,
+                                     const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
+                                     const float *q_norm_w, const float *k_norm_w, float eps,
+                                     float attn_scalar, float *out_dev) {
+    if (!L || !qg_dev || !k_dev || !v_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step_gated: pointeur nul");
+    if ((qg_off | k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "decode_step_gated: offset non aligné f32");
+    // split_q_gate (src/decode_resident/kernels.rs:931-946) by addressing: head h holds its
+    // head_dim query values at h * 2 * head_dim and its gate values right after them
+    const float *qg = reinterpret_cast<const float *>((const char *)qg_dev + qg_off);
+    const size_t hd = (size_t)L->g.head_dim;
+    return prekv_step(L, stream, rope, position, qg, 2 * hd, qg + hd,
+                      reinterpret_cast<const float *>((const char *)k_dev + k_off),
+                      reinterpret_cast<const float *>((const char *)v_dev + v_off), q_norm_w,
+                      k_norm_w, eps, attn_scalar, out_dev);
+}
+
+int32_t skv_attn_gate_device(skv_ctx *ctx, skv_stream stream, const float *ctx_dev, const float *gate_dev,
+                             size_t gate_head_stride, size_t heads, size_t head_dim, float *out_dev) {
+    if (!ctx || !ctx_dev || !gate_dev || !out_dev) return fail(SKV_ERR_DEVICE, "attn_gate: pointeur nul");
+    if (heads == 0 || head_dim == 0 || heads * head_dim > ((size_t)1 << 30))
+        return fail(SKV_ERR_DIMENSION, "attn_gate: dimensions invalides");
+    if (gate_head_stride != 0 && gate_head_stride < head_dim)
+        return fail(SKV_ERR_DIMENSION, "attn_gate: pas du gate < head_dim");
+    GateArgs ga{};
+    ga.ctx = ctx_dev;
+    ga.gate = gate_dev;
+    ga.out = out_dev;
+    ga.heads = (int)heads;
+    ga.head_dim = (int)head_dim;
+    ga.gate_head_stride = (int)(gate_head_stride ? gate_head_stride : head_dim);
+    SKV_HIP(launch_gate(ga, as_stream(stream)));
+    return SKV_OK;
 }
 
 int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_stream stream,

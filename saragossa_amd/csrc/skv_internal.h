@@ -118,6 +118,10 @@ struct DecodeArgs {
     const float *rope;      // [rope_dims/2][2]: (cos, sin) of this position
     const float *q_norm_w;  // [head_dim]
     const float *k_norm_w;  // [head_dim]
+    // decode only: head h of q starts at q + h * q_head_stride (0 = head_dim), and the
+    // context of head h is multiplied by sigmoid(gate[h * q_head_stride + col]) (null = none)
+    const float *gate;
+    int q_head_stride;
     Geom g;
 };
 static_assert(sizeof(DecodeArgs) <= 256, "sixteen of them must fit the kernel argument block");
@@ -130,10 +134,22 @@ struct NormRopeArgs {
     const float *rope;   // [rope_dims/2][2] or null
     int heads, head_dim, rope_dims, rope_style;
     float eps;
+    int x_head_stride; // elements between the heads of x (0 = head_dim)
 };
+
+// out[h][c] = ctx[h][c] * sigmoid(gate[h * gate_head_stride + c])
+struct GateArgs {
+    const float *ctx;
+    const float *gate;
+    float *out;
+    int heads, head_dim, gate_head_stride;
+};
+hipError_t launch_gate(const GateArgs &a, hipStream_t s);
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s);
 
 #ifdef __HIPCC__
+// sigmoid_scalar (src/decoder/attention_ops.rs:522-524)
+__device__ __forceinline__ float sigmoid_gate(float g) { return 1.0f / (1.0f + expf(-g)); }
 // The arithmetic of rms_norm_rope_heads_at (src/decoder/attention_ops.rs:682-777), operation
 // for operation and without contraction, so that the device row equals the CPU row bit for
 // bit when the (cos, sin) table comes from the host's libm.

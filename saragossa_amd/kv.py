@@ -72,6 +72,12 @@ class DecodeResidentState:
                                                     _p(out)))
         return out
 
+    def encode_attn_gate(self, stream, ctx_ptr, gate_ptr, gate_head_stride, heads, head_dim,
+                         out_ptr) -> None:
+        """encode_attn_gate (attn_gate_f32, src/decode_resident/kernels.rs:949-959)."""
+        check(self._l.skv_attn_gate_device(self._h, stream, ctx_ptr, gate_ptr, gate_head_stride,
+                                           heads, head_dim, out_ptr))
+
     def rope_table(self, max_positions, rope_dims, theta, position_scale=1.0, frequency_dim=0,
                    style=0) -> "RopeTable":
         return RopeTable(self, max_positions, rope_dims, theta, position_scale, frequency_dim, style)
@@ -227,6 +233,14 @@ class FullAttentionState:
         encode_resident_full_layer (src/decode_resident/layers.rs:214-288) in one call."""
         check(self._l.skv_decode_step_prekv_device(
             self._h, stream, None if rope is None else rope._h, position, q_ptr, q_off, k_ptr,
+            k_off, v_ptr, v_off, q_norm_ptr, k_norm_ptr, eps, attn_scalar, out_ptr))
+
+    def encode_decode_step_gated(self, stream, rope, position, qg_ptr, qg_off, k_ptr, k_off, v_ptr,
+                                 v_off, q_norm_ptr, k_norm_ptr, eps, attn_scalar, out_ptr) -> None:
+        """encode_decode_step_prekv for a layer with an output gate: qg is the gated q
+        projection (per head: q then gate) and the context comes out times sigmoid(gate)."""
+        check(self._l.skv_decode_step_gated_device(
+            self._h, stream, None if rope is None else rope._h, position, qg_ptr, qg_off, k_ptr,
             k_off, v_ptr, v_off, q_norm_ptr, k_norm_ptr, eps, attn_scalar, out_ptr))
 
     def encode_gather(self, stream, first, n, k_dst_ptr, v_dst_ptr) -> None:

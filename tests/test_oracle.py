@@ -323,3 +323,27 @@ def test_attention_layout_rules():
         args.update(bad)
         with pytest.raises(oracle.OracleError):
             oracle.attention_layout(**args)
+
+
+def test_output_gate_split_and_sigmoid():
+    """split_attention_gate + sigmoid gate (src/decoder/attention_ops.rs:486-524, 217-219)."""
+    heads, hd, rows = 3, 4, 2
+    qp = np.arange(rows * heads * 2 * hd, dtype=np.float32).reshape(rows, -1)
+    q, gate = oracle.split_attention_gate(qp, heads, hd)
+    r = qp.reshape(rows, heads, 2, hd)
+    assert np.array_equal(q, r[:, :, 0].reshape(rows, -1))
+    assert np.array_equal(gate, r[:, :, 1].reshape(rows, -1))
+    with pytest.raises(oracle.OracleError):
+        oracle.split_attention_gate(qp[:, :-1], heads, hd)
+    ctx = np.float32([2.0, -3.0, 0.5, 1.0, 7.0])
+    g = np.float32([0.0, 0.0, 30.0, -30.0, -200.0])
+    out = oracle.attention_gate(ctx, g)
+    assert out[0] == 1.0 and out[1] == -1.5             # sigmoid(0) is exactly 1/2
+    assert out[2] == 0.5                                # saturates to 1
+    assert 0.0 < out[3] < 1e-12 and out[4] == 0.0       # exp overflows to inf: 1/inf == 0
+    x = np.linspace(-20, 20, 4001).astype(np.float32)
+    one = np.ones_like(x)
+    s_pos, s_neg = oracle.attention_gate(one, x), oracle.attention_gate(one, -x)
+    assert np.abs(s_pos + s_neg - 1.0).max() <= 2e-7
+    want = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    assert np.abs(s_pos - want).max() <= 1.2e-7         # within an ulp or so of the fp64 value

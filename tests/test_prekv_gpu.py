@@ -210,3 +210,92 @@ def test_prekv_errors(state):
     step(rope, 0)
     step(None, 1)                     # no rotation at all
     assert kv.len() == 2
+
+
+# ---- output gate -------------------------------------------------------------------------
+
+def test_attn_gate_matches_cpu(state):
+    """encode_attn_gate (attn_gate_f32) against context * sigmoid_scalar(gate); the gate may sit
+    interleaved with q in the gated projection."""
+    heads, hd = 16, 256
+    rng = np.random.default_rng(3)
+    ctx = rng.standard_normal(heads * hd, dtype=np.float32)
+    qg = rng.standard_normal(heads * 2 * hd, dtype=np.float32) * 4
+    _, gate = oracle.split_attention_gate(qg, heads, hd)
+    want = oracle.attention_gate(ctx, gate[0])
+    cd, gd = _dev(ctx), _dev(qg)
+    out = torch.empty(heads * hd, device="cuda", dtype=torch.float32)
+    state.encode_attn_gate(_stream(), cd.data_ptr(), gd.data_ptr() + hd * 4, 2 * hd, heads, hd,
+                           out.data_ptr())
+    assert np.abs(out.cpu().numpy() - want).max() <= 1e-6
+    # contiguous gate, in place
+    g2 = _dev(gate[0])
+    state.encode_attn_gate(_stream(), cd.data_ptr(), g2.data_ptr(), 0, heads, hd, cd.data_ptr())
+    assert np.abs(cd.cpu().numpy() - want).max() <= 1e-6
+
+
+GATED = [
+    ((16, 2, 256), 0, 700, 30, 64, 1.0e7),    # config 2's full-attention layers (gated, partial rotary), split-K
+    ((16, 2, 256), 0, 3, 30, 64, 1.0e7),      # short cache: the split kernel applies the gate itself
+    ((8, 4, 64), 32, 5, 80, 64, 10000.0),     # ring layer
+    ((6, 2, 96), 0, 40, 10, 48, 10000.0),     # padded head_dim
+]
+
+
+def run_gated(state, dims, window, start, steps, rope_dims, theta):
+    q_heads, kv_heads, head_dim = dims
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    eps = 1.0e-6
+    rng = np.random.default_rng(start * 5 + steps)
+    cap = start + steps
+    kv = state.full_attention_bf16(cap, q_heads, kv_heads, head_dim, window=window)
+    kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r")
+    q_norm = (0.7 + np.abs(pseudo(np.arange(head_dim) * 11))).astype(np.float32)
+    k_norm = (0.8 + np.abs(pseudo(np.arange(head_dim) * 17))).astype(np.float32)
+    if start:
+        k0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+        v0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+        kv.seed(k0, v0, start)
+        cache.append_batch(k0, v0, lay)
+    rope = state.rope_table(cap, rope_dims, theta)
+    # gated q projection | k | v, as the fused projection leaves them
+    raw = rng.standard_normal((steps, 2 * q_dim + 2 * kv_dim), dtype=np.float32) * 1.5
+    rd, qwd, kwd = _dev(raw), _dev(q_norm), _dev(k_norm)
+    out = torch.empty(steps, q_dim, device="cuda", dtype=torch.float32)
+    for t in range(steps):
+        kv.encode_decode_step_gated(
+            _stream(), rope, start + t, rd[t].data_ptr(), 0, rd[t].data_ptr(), 2 * q_dim * 4,
+            rd[t].data_ptr(), (2 * q_dim + kv_dim) * 4, qwd.data_ptr(), kwd.data_ptr(), eps,
+            float(head_dim), out[t].data_ptr())
+    got = out.cpu().numpy()
+    worst = 0.0
+    for t in range(steps):
+        pos = start + t
+        q_raw, gate = oracle.split_attention_gate(raw[t, :2 * q_dim], q_heads, head_dim)
+        q_cpu = oracle.rms_norm_rope_heads_at(q_raw[0], q_heads, head_dim, rope_dims, q_norm, eps, theta, pos)[0]
+        k_cpu = oracle.rms_norm_rope_heads_at(raw[t, 2 * q_dim:2 * q_dim + kv_dim], kv_heads, head_dim,
+                                              rope_dims, k_norm, eps, theta, pos)[0]
+        ctx = oracle.decode_step(cache, k_cpu, raw[t, 2 * q_dim + kv_dim:], q_cpu, lay)
+        want = oracle.attention_gate(ctx, gate[0])
+        worst = max(worst, float(np.abs(got[t] - want).max()))
+    assert worst <= 1e-4, worst
+    first = 0 if window == 0 else max(0, cap - (window + 15) // 16 * 16)
+    gk, gv = kv.read_rows_f32(first, cap - first)
+    assert np.array_equal(gk, cache.keys()[first:]) and np.array_equal(gv, cache.values()[first:])
+    rope.close()
+
+
+@pytest.mark.parametrize("dims,window,start,steps,rope_dims,theta", GATED)
+def test_gated_steps_match_oracle(state, dims, window, start, steps, rope_dims, theta):
+    """The Qwen3.5/3.6 full-attention block from the gated q projection to the o projection's
+    input: split, norms, rotation, append, attention, sigmoid gate."""
+    run_gated(state, dims, window, start, steps, rope_dims, theta)
+
+
+@pytest.mark.parametrize("dims,window,start,steps,rope_dims,theta", [GATED[0], GATED[2]])
+def test_gated_steps_as_separate_launches(state, env_flags, dims, window, start, steps, rope_dims,
+                                          theta):
+    env_flags(RETI_RUST_FLASH_SDPA="0")
+    run_gated(state, dims, window, start, steps, rope_dims, theta)
