@@ -1,0 +1,70 @@
+"""Speculative decoding at the KV boundary: k draft rows are verified in one multi-query
+launch over the cache (the per-row loop of the resident verify, src/decoder/resident/
+verify.rs:157-203, as one call), then the cache is rolled back to the accepted length with
+truncate (restore_mtp_resident_progress, src/decoder/generation.rs:1026-1064). After the
+rollback the layer must behave as if the rejected rows had never been appended."""
+import numpy as np
+import pytest
+
+import oracle
+import saragossa_amd as skv
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.mark.parametrize("dims,window,base,rounds", [
+    ((16, 2, 256), 0, 700, 6),      # full layer, split-K
+    ((32, 8, 128), 0, 40, 8),       # short cache
+    ((8, 2, 64), 20, 100, 10),      # ring of 32 rows for a window of 20: 12 rows of slack
+])
+def test_verify_rows_then_rollback_equals_never_appended(state, dims, window, base, rounds):
+    q_heads, kv_heads, head_dim = dims
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(base + rounds)
+    k_draft = 5
+    cap = base + rounds * k_draft + 8
+    kv = state.full_attention_bf16(cap, q_heads, kv_heads, head_dim, window=window)
+    kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r")
+    k0 = rng.standard_normal((base, kv_dim), dtype=np.float32)
+    v0 = rng.standard_normal((base, kv_dim), dtype=np.float32)
+    kv.seed(k0, v0, base)
+    cache.append_batch(k0, v0, lay)
+    for r in range(rounds):
+        q = rng.standard_normal((k_draft, q_dim), dtype=np.float32)
+        k = rng.standard_normal((k_draft, kv_dim), dtype=np.float32)
+        v = rng.standard_normal((k_draft, kv_dim), dtype=np.float32)
+        start = kv.len()
+        got = kv.prefill_rows(q, k, v)                       # verify the k draft rows at once
+        accepted = int(rng.integers(1, k_draft + 1))         # at least the first row is kept
+        # the oracle only ever sees the accepted rows, one by one
+        want = oracle.cached_attention_prefill_rows(q[:accepted], k[:accepted], v[:accepted], cache, lay)
+        assert np.abs(got[:accepted] - want).max() <= 1e-4
+        kv.truncate(start + accepted)                        # rollback
+        assert kv.len() == len(cache) == start + accepted
+    # after all the rollbacks: contents and a decode step agree with the oracle
+    first = 0 if window == 0 else max(0, kv.len() - window)
+    gk, gv = kv.read_rows_f32(first, kv.len() - first)
+    assert np.array_equal(gk, cache.keys()[first:]) and np.array_equal(gv, cache.values()[first:])
+    q = rng.standard_normal(q_dim, dtype=np.float32)
+    ws = skv.flags.window_start(kv.len() - 1, window)
+    assert np.abs(kv.attention_decode_windowed(q, ws) - oracle.cached_attention_one(q, cache, lay)).max() <= 1e-4
+
+
+def test_rollback_on_a_ring_without_slack_is_an_error_not_stale_data(state):
+    """A ring that holds exactly its window has overwritten the rows a rollback would need:
+    the next attention reports it."""
+    q_heads, kv_heads, head_dim, window = 8, 2, 64, 32
+    kv_dim = kv_heads * head_dim
+    rng = np.random.default_rng(4)
+    kv = state.full_attention_bf16(200, q_heads, kv_heads, head_dim, window=window)
+    k = rng.standard_normal((100, kv_dim), dtype=np.float32)
+    kv.seed(k, k, 100)
+    q = rng.standard_normal((4, q_heads * head_dim), dtype=np.float32)
+    kv.prefill_rows(q, k[:4], k[:4])
+    kv.truncate(101)
+    with pytest.raises(skv.DimensionError):
+        kv.attention_decode_windowed(q[0], skv.flags.window_start(100, window))
