@@ -644,6 +644,10 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     default: break;
     }
     if (e != hipSuccess || a.splits == 1) return e;
+    return launch_merge(a, s);
+}
+
+hipError_t launch_merge(const DecodeArgs &a, hipStream_t s) {
     dim3 mgrid((unsigned)(a.g.kv_heads * a.n_queries * a.g.gqa), (unsigned)((a.g.head_dim + 15) / 16));
     const int per_lane = (a.splits + 15) / 16;
     if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_kernel<1>, mgrid, dim3(256), 0, s, a);

@@ -127,6 +127,7 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
     a.k_pool_w = L->k_pool;
     a.v_pool_w = L->v_pool;
     a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
+    a.q_vec = ((reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
     a.g = g;
 }
 
@@ -197,11 +198,18 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
         a.gate = pre->gate;
         a.q_head_stride = pre->q_head_stride;
     }
+    // Chunks of at least 64 query slots take the kernel that shares each K/V page among 128
+    // or 256 slots through LDS; shorter ones (speculative verify rows) the decode kernel's
+    // multi-query mode, one workgroup per 16 slots.
+    static const bool tiles_enabled = env_usize("SKV_PREFILL_TILES", 1) != 0;
+    const bool use_tiles = tiles_enabled && n_queries > 1 && n_queries * (size_t)g.gqa >= 64;
     if (n_queries > 1) {
-        // every 16 query slots are a workgroup of their own: split the context only while
-        // that leaves compute units idle, and keep the partials in the context's scratch
-        const size_t tiles = (n_queries * (size_t)g.gqa + 15) / 16 * (size_t)g.kv_heads;
-        const size_t want = std::max<size_t>(256 / tiles, 1);
+        // split the context only while the query tiles alone leave compute units idle, and
+        // keep the partials in the context's scratch
+        const size_t per_wg = use_tiles ? (size_t)prefill_tile_slots(g.P) : 16;
+        const size_t tiles = (n_queries * (size_t)g.gqa + per_wg - 1) / per_wg * (size_t)g.kv_heads;
+        size_t want = std::max<size_t>(256 / tiles, 1);
+        if (use_tiles) want = std::min<size_t>(want, std::max<size_t>((size_t)a.n_pages / 16, 1));
         a.splits = (int)std::min<size_t>((size_t)a.splits, want);
         if (a.splits > 1) {
             const size_t n_part = (size_t)g.kv_heads * a.splits * n_queries * g.gqa;
@@ -219,6 +227,11 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
             a.part_m = a.part_o + n_part * g.head_dim;
             a.part_l = a.part_m + n_part;
         }
+    }
+    if (use_tiles) {
+        SKV_HIP(launch_prefill_tiles(a, s));
+        if (a.splits > 1) SKV_HIP(launch_merge_rows(a, s));
+        return SKV_OK;
     }
     SKV_HIP(launch_decode(a, s));
     return SKV_OK;

@@ -122,6 +122,7 @@ struct DecodeArgs {
     // context of head h is multiplied by sigmoid(gate[h * q_head_stride + col]) (null = none)
     const float *gate;
     int q_head_stride;
+    int q_vec;              // q is 16-byte aligned and head_dim a multiple of 8: 16-byte loads
     Geom g;
 };
 static_assert(sizeof(DecodeArgs) <= 256, "sixteen of them must fit the kernel argument block");
@@ -239,6 +240,10 @@ hipError_t launch_append(const AppendArgs &a, hipStream_t s);
 hipError_t launch_gather(const GatherArgs &a, hipStream_t s);
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s);
 hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s);
+hipError_t launch_merge(const DecodeArgs &a, hipStream_t s);        // split-K partials -> context
+hipError_t launch_prefill_tiles(const DecodeArgs &a, hipStream_t s); // chunked prefill, no merge
+int prefill_tile_slots(int P);
+hipError_t launch_merge_rows(const DecodeArgs &a, hipStream_t s);    // the same merge for many query slots
 hipError_t launch_naive(const NaiveArgs &a, hipStream_t s);
 int decode_max_splits();
 
