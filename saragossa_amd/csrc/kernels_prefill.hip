@@ -29,14 +29,15 @@ __device__ __forceinline__ float xor_max(float v, int mask) { return fmaxf(v, __
 //
 // One workgroup = 8 wavefronts = 8 * TILES tiles of 16 query slots of one kv head, and a
 // range of the context's pages (split). The workgroup walks its pages once: all threads
-// copy the page's K and V tiles (already in matrix-operand order) from memory to LDS, double
+// copy PG pages' K and V tiles (already in matrix-operand order) from memory to LDS, double
 // buffered, and every wavefront multiplies them with its own query tiles, which it holds in
 // registers as bf16 hi + lo halves (pre-scaled by log2(e)/sqrt(head_dim)). So a K/V byte is
-// fetched from memory once per 128 * TILES query slots instead of once per 16. Per page and
-// tile: S^T = K . Q^T (16 keys x 16 slots), online softmax in base 2 on the accumulator
-// registers, O^T += V^T . P^T with P split hi + lo. There is no merge inside the workgroup
-// (every wavefront owns its slots); with several splits the (o, m, l) partials go to the
-// same merge kernel as decode.
+// fetched from memory once per 128 * TILES query slots instead of once per 16. Pages are
+// consumed in pairs: S^T = K . Q^T per page (16 keys x 16 slots, 16x16x32 over the head
+// dims), one online-softmax step in base 2 over the pair's 32 keys on the accumulator
+// registers, then O^T += V^T . P^T as 16x16x32 products over those 32 keys with P split
+// hi + lo. There is no merge inside the workgroup (every wavefront owns its slots); with
+// several splits the (o, m, l) partials go to merge_rows_kernel.
 // ------------------------------------------------------------------------------------
 // Copies of PG pages (K tile then V tile each) of one kv head: memory -> registers -> LDS.
 template <int P, int PG>
@@ -134,32 +135,39 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
         t_ws_lo[t] = ws_of(t_lim_lo[t]);
         t_ws_hi[t] = ws_of(t_lim_hi[t]);
         const float *qrow = a.q + ((long)(my_slot / G) * g.q_heads + kvh * G + my_slot % G) * g.head_dim;
+        // eight consecutive dims of the slot's row per k-step: all loads first (two 16-byte
+        // loads per step when the row allows), unconditional from clamped addresses, so that
+        // they are one round trip; dims past head_dim are zeroed afterwards
+        float qv[KK][8];
+        if (a.q_vec) {
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            // eight consecutive dims of the slot's row: two 16-byte loads when the row allows
-            float qv[8];
-            const int d0 = kk * 32 + j * 8;
-            if (a.q_vec) {
-                const float4_t z = {0.f, 0.f, 0.f, 0.f};
+            for (int kk = 0; kk < KK; ++kk) {
+                const int d0 = kk * 32 + j * 8;
                 const float4_t *qp = reinterpret_cast<const float4_t *>(qrow + min(d0, g.head_dim - 8));
-                const float4_t x0 = d0 < g.head_dim ? qp[0] : z;
-                const float4_t x1 = d0 < g.head_dim ? qp[1] : z;
+                const float4_t x0 = qp[0], x1 = qp[1];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    qv[e] = x0[e];
-                    qv[4 + e] = x1[e];
+                    qv[kk][e] = x0[e];
+                    qv[kk][4 + e] = x1[e];
                 }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) qv[e] = d0 + e < g.head_dim ? qrow[min(d0 + e, g.head_dim - 1)] : 0.0f;
             }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qv[kk][e] = qrow[min(kk * 32 + j * 8 + e, g.head_dim - 1)];
+            }
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const int d0 = kk * 32 + j * 8;
             uint32_t hi[4], lo[4];
 #pragma unroll
             for (int e2 = 0; e2 < 4; ++e2) {
                 uint32_t h2 = 0, l2 = 0;
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const float v = qv[e2 * 2 + h] * a.qscale;
+                    const float v = d0 + e2 * 2 + h < g.head_dim ? qv[kk][e2 * 2 + h] * a.qscale : 0.0f;
                     const uint16_t hb = bf16_bits(v);
                     const uint16_t lb = bf16_bits(v - bf16_to_f32(hb));
                     h2 |= (uint32_t)hb << (16 * h);
@@ -405,7 +413,7 @@ hipError_t launch_merge_rows(const DecodeArgs &a, hipStream_t s) {
 }
 
 // Query slots one workgroup of the kernel covers for a padded head_dim.
-int prefill_tile_slots(int P) { return P <= 128 ? 256 : 128; }
+int prefill_tile_slots(int P) { return P <= 64 ? 256 : 128; }
 
 template <int P, int TILES, int PG>
 static hipError_t launch_tiles(const DecodeArgs &a, dim3 grid, hipStream_t s) {
@@ -428,7 +436,7 @@ hipError_t launch_prefill_tiles(const DecodeArgs &a, hipStream_t s) {
     switch (a.g.P) {
     case 32: return launch_tiles<32, 2, 8>(a, grid, s);
     case 64: return launch_tiles<64, 2, 8>(a, grid, s);
-    case 128: return launch_tiles<128, 2, 8>(a, grid, s);
+    case 128: return launch_tiles<128, 1, 8>(a, grid, s);
     case 256: return launch_tiles<256, 1, 4>(a, grid, s);
     default: return hipErrorInvalidValue;
     }

@@ -208,8 +208,11 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
         // keep the partials in the context's scratch
         const size_t per_wg = use_tiles ? (size_t)prefill_tile_slots(g.P) : 16;
         const size_t tiles = (n_queries * (size_t)g.gqa + per_wg - 1) / per_wg * (size_t)g.kv_heads;
-        size_t want = std::max<size_t>(256 / tiles, 1);
-        if (use_tiles) want = std::min<size_t>(want, std::max<size_t>((size_t)a.n_pages / 16, 1));
+        size_t want = std::max<size_t>((use_tiles ? env_usize("SKV_PREFILL_WGS", 256) : 256) / tiles, 1);
+        if (use_tiles) {
+            want = std::min<size_t>(want, std::max<size_t>((size_t)a.n_pages / 16, 1));
+            want = std::min<size_t>(want, std::max<size_t>(env_usize("SKV_PREFILL_MAX_SPLITS", 512), 1));
+        }
         a.splits = (int)std::min<size_t>((size_t)a.splits, want);
         if (a.splits > 1) {
             const size_t n_part = (size_t)g.kv_heads * a.splits * n_queries * g.gqa;
