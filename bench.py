@@ -150,6 +150,53 @@ def bench_restore(skv, torch, np, state, stream):
     return out
 
 
+def bench_prefill(skv, torch, np, state, stream):
+    """Chunked prefill over the cache (cached_attention_prefill_rows as one launch): a
+    512-row chunk appended and attended causally over the rows already cached, at the KV
+    shapes of configs[2] (after 32768 rows) and configs[1] (the last chunk of its 2048-token
+    prompt). The one matrix-core-bound kernel of the path: flops = 4 * keys * q_dim over the
+    (query, key) pairs attended; the kernel issues twice that on the matrix cores because
+    queries and probabilities are split into two bf16 terms."""
+    dev = torch.device("cuda:0")
+    out = []
+    for name, (qh, kvh, hd), base, chunk in (("configs[2] shape q16/kv2/hd256", (16, 2, 256), 32768, 512),
+                                            ("configs[1] shape q32/kv8/hd128", (32, 8, 128), 1536, 512)):
+        kv_dim, q_dim = kvh * hd, qh * hd
+        kv = state.full_attention_bf16(base + chunk + 16, qh, kvh, hd)
+        kv.set_block_table(np.random.default_rng(7).permutation(kv.pages()).astype(np.int32))
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(7)
+        k0 = torch.randn(base, kv_dim, device=dev, generator=gen)
+        v0 = torch.randn(base, kv_dim, device=dev, generator=gen)
+        kv.encode_append_batch(stream, k0.data_ptr(), v0.data_ptr(), base)
+        q = torch.randn(chunk, q_dim, device=dev, generator=gen)
+        k = torch.randn(chunk, kv_dim, device=dev, generator=gen)
+        v = torch.randn(chunk, kv_dim, device=dev, generator=gen)
+        o = torch.empty(chunk, q_dim, device=dev)
+        ts = []
+        for it in range(13):
+            kv.truncate(base)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            kv.encode_prefill_rows(stream, q.data_ptr(), k.data_ptr(), v.data_ptr(), chunk, o.data_ptr())
+            e1.record()
+            torch.cuda.synchronize()
+            if it >= 3:
+                ts.append(e0.elapsed_time(e1) * 1e3)
+        ts.sort()
+        us = ts[len(ts) // 2]
+        keys = sum(base + i + 1 for i in range(chunk))
+        flops = 4 * keys * q_dim
+        out.append({"workload": "%s: %d-row chunk over %d cached rows (append + attention + merge)"
+                                % (name, chunk, base),
+                    "us": round(us, 1), "algorithmic_tflops": round(flops / us / 1e6, 1),
+                    "mfma_tflops_issued": round(2 * flops / us / 1e6, 1),
+                    "frac_of_bf16_mfma_peak": round(2 * flops / us / 1e6 / 2500.0, 4)})
+        kv.close()
+    return out
+
+
 class _TimedHot:
     """HotCache with HIP events around the calls the serve path makes, so that the restore and
     snapshot legs of a turn can be told apart afterwards."""
@@ -579,6 +626,8 @@ def main() -> int:
         result["restore"] = restore
     if recurrent is not None:
         result["recurrent_state"] = recurrent
+    if args.config == 2 and not args.no_restore:
+        result["prefill"] = bench_prefill(skv, torch, np, state, stream)
 
     if not args.no_cpu_baseline:
         import oracle
