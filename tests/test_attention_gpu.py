@@ -201,6 +201,12 @@ def test_normal_inputs_config0(state):
     ((16, 2, 256), 5, 3, 0),         # speculative-verify sized chunk (split over the context)
     ((4, 2, 16), 0, 50, 0),
     ((6, 1, 40), 17, 33, 0),         # head_dim padded to 64, GQA 6
+    # chunks of 64 query slots and more take the kernel that shares K/V pages through LDS
+    ((16, 2, 256), 5000, 600, 0),    # several workgroups per kv head, split context, ragged tail
+    ((32, 8, 128), 0, 1000, 0),      # from an empty cache: early tiles see few pages (empty splits)
+    ((6, 1, 40), 100, 100, 0),       # rows too short for 16-byte query loads, padded head_dim
+    ((8, 1, 32), 33, 77, 0),         # head_dim 32, odd page count
+    ((40, 1, 64), 10, 9, 0),         # GQA 40: 360 slots from 9 rows
 ])
 def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk, window):
     """One launch == the reference's per-row loop (append, then cached_attention_one)."""
@@ -227,11 +233,15 @@ def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk, window):
     assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
 
 
-@pytest.mark.parametrize("window,chunks", [(32, [40, 7, 64]), (20, [5, 30, 3])])
-def test_prefill_rows_on_ring_layer(state, window, chunks):
+@pytest.mark.parametrize("window,chunks,heads", [
+    (32, [40, 7, 64], (8, 2)), (20, [5, 30, 3], (8, 2)),
+    (250, [7, 300, 20], (32, 2)),   # 7-row steps of 16 heads per group: the LDS-shared kernel on a ring
+    (100, [130, 50], (64, 4)),
+])
+def test_prefill_rows_on_ring_layer(state, window, chunks, heads):
     """A ring that holds exactly its window advances row by row; results equal the oracle's
     sliding-window attention."""
-    q_heads, kv_heads, head_dim = 8, 2, 64
+    (q_heads, kv_heads), head_dim = heads, 64
     kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
     rng = np.random.default_rng(window)
     lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)

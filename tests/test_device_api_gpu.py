@@ -241,3 +241,34 @@ def test_decode_step_batch_errors(state):
     torch.cuda.synchronize()
     assert a.len() == 1 and b.len() == 1
     assert np.array_equal(out.cpu().numpy(), np.zeros((2, 8 * 64), np.float32))  # one key: out == its V row
+
+
+def test_prefill_chunk_device_with_unaligned_query_pointer(state):
+    """The chunk's q rows may start at any 4-byte offset of a larger buffer: the kernel then
+    takes the 4-byte query loads."""
+    q_heads, kv_heads, head_dim, start, chunk = 16, 2, 128, 200, 40
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(77)
+    lay = oracle.layout(q_heads, kv_heads, head_dim)
+    results = []
+    for pad in (0, 1, 3):
+        kv = state.full_attention_bf16(start + chunk, q_heads, kv_heads, head_dim)
+        cache = oracle.LayerKvCache("bf16r")
+        r2 = np.random.default_rng(78)
+        k0 = r2.standard_normal((start, kv_dim), dtype=np.float32)
+        v0 = r2.standard_normal((start, kv_dim), dtype=np.float32)
+        kv.seed(k0, v0, start)
+        cache.append_batch(k0, v0, lay)
+        q = r2.standard_normal((chunk, q_dim), dtype=np.float32)
+        k = r2.standard_normal((chunk, kv_dim), dtype=np.float32)
+        v = r2.standard_normal((chunk, kv_dim), dtype=np.float32)
+        buf = _dev(np.concatenate([np.zeros(pad, np.float32), q.reshape(-1)]))
+        kd, vd = _dev(k), _dev(v)
+        out = torch.empty(chunk, q_dim, device="cuda", dtype=torch.float32)
+        kv.encode_prefill_rows(_stream(), buf.data_ptr() + pad * 4, kd.data_ptr(), vd.data_ptr(), chunk,
+                               out.data_ptr())
+        got = out.cpu().numpy()
+        want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+        assert np.abs(got - want).max() <= 1e-4
+        results.append(got)
+    assert np.array_equal(results[0], results[1]) and np.array_equal(results[0], results[2])
