@@ -188,8 +188,18 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         const int qs = min(tile * 16 + (idx & 15), n_slots - 1);
         const float *qrow = MQ ? a.q + ((long)(qs / G) * g.q_heads + kvh * G + qs % G) * g.head_dim
                                : a.q + (long)(kvh * G + qs) * q_stride;
+        if (a.q_vec) { // two 16-byte loads from a clamped address (dims past head_dim are zeroed below)
+            const float4_t *qp = reinterpret_cast<const float4_t *>(qrow + min(kk * 32 + jj * 8, g.head_dim - 8));
+            const float4_t x0 = qp[0], x1 = qp[1];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qv[u][e] = qrow[min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
+            for (int e = 0; e < 4; ++e) {
+                qv[u][e] = x0[e];
+                qv[u][4 + e] = x1[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qv[u][e] = qrow[min(kk * 32 + jj * 8 + e, g.head_dim - 1)];
+        }
     }
     // Unconditional (a wavefront without pages reads physical page 0 and ignores it): a
     // conditional load here makes the compiler wait for these pages before the queries.
@@ -610,13 +620,10 @@ static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     const int rows = n_slots < 16 ? n_slots : 16;
     const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
     const size_t lds = stage > xchg ? stage : xchg;
-    static bool attr_set = false; // per instantiation
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES, MQ, PRE>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static std::atomic<uint64_t> lds_ok{0}; // per instantiation
+    {
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES, MQ, PRE>), lds_ok);
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
     hipLaunchKernelGGL((decode_split_kernel<P, WAVES, MQ, PRE>), grid, dim3(WAVES * 64), lds, s, a);
@@ -667,13 +674,10 @@ static hipError_t launch_split_batch(const DecodeBatchArgs &b, int n_seq, int ma
     const int rows = g.gqa < 16 ? g.gqa : 16;
     const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
     const size_t lds = stage > xchg ? stage : xchg;
-    static bool attr_set = false; // per instantiation
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&decode_split_batch_kernel<P, WAVES>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static std::atomic<uint64_t> lds_ok{0}; // per instantiation
+    {
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&decode_split_batch_kernel<P, WAVES>), lds_ok);
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     dim3 grid((unsigned)max_splits, (unsigned)g.kv_heads, (unsigned)n_seq);
     hipLaunchKernelGGL((decode_split_batch_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, b);

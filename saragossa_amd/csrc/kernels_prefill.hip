@@ -418,12 +418,10 @@ int prefill_tile_slots(int P) { return P <= 64 ? 256 : 128; }
 template <int P, int TILES, int PG>
 static hipError_t launch_tiles(const DecodeArgs &a, dim3 grid, hipStream_t s) {
     constexpr size_t lds = (size_t)2 * PG * 2 * (P / 32) * 64 * sizeof(uint4);
-    static bool attr_set = false; // per instantiation
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_tile_kernel<P, TILES, PG>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static std::atomic<uint64_t> lds_ok{0}; // per instantiation
+    {
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&prefill_tile_kernel<P, TILES, PG>), lds_ok);
         if (e != hipSuccess) return e;
-        attr_set = true;
     }
     hipLaunchKernelGGL((prefill_tile_kernel<P, TILES, PG>), grid, dim3(512), lds, s, a);
     return hipGetLastError();

@@ -127,7 +127,8 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
     a.k_pool_w = L->k_pool;
     a.v_pool_w = L->v_pool;
     a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
-    a.q_vec = ((reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
+    static const bool q_vec_enabled = env_usize("SKV_Q_VEC", 1) != 0;
+    a.q_vec = (q_vec_enabled && (reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
     a.g = g;
 }
 

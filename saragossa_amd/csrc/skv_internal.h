@@ -1,6 +1,7 @@
 // Internal declarations shared by the host side and the kernel launchers.
 #pragma once
 
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -147,6 +148,20 @@ struct GateArgs {
 };
 hipError_t launch_gate(const GateArgs &a, hipStream_t s);
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s);
+
+// Raises a kernel's dynamic LDS limit to the 160 KiB of a gfx950 compute unit, once per
+// device and kernel (`done` is a per-kernel bit mask over device ids; the attribute belongs to
+// the current device's copy of the code object).
+inline hipError_t allow_full_lds(const void *kernel, std::atomic<uint64_t> &done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+    return e;
+}
 
 #ifdef __HIPCC__
 // sigmoid_scalar (src/decoder/attention_ops.rs:522-524)

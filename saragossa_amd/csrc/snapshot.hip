@@ -681,7 +681,9 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
                             pages.size(), nullptr, false, as_stream(stream));
             if (rc) return rc;
             done_blocks = chain.size();
-            batch = std::min<size_t>(batch * 2, COPY_MAX_PAGES);
+            // a copy of b pages takes about 2.4 times as long as hashing b blocks, so the next
+            // batch may be that much larger without the queue running dry
+            batch = std::min<size_t>(batch * 5 / 2, COPY_MAX_PAGES);
         }
         if (!walk.alive) break;
     }
