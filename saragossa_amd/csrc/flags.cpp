@@ -161,6 +161,17 @@ size_t skv_flag_prefill_chunk(void) {
     });
 }
 
+} // extern "C"
+
+// Generation of the cached flag values: callers that cache their own environment-derived
+// settings re-read them when it changes.
+uint64_t skv_internal_flags_epoch() {
+    std::lock_guard<std::mutex> lk(g_mu);
+    return g_epoch;
+}
+
+extern "C" {
+
 void skv_flags_reload(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     ++g_epoch;

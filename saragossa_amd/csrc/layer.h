@@ -39,3 +39,5 @@ struct skv_layer {
     size_t scores_cap = 0;
 };
 
+// flags.cpp: generation counter of the cached runtime flags
+uint64_t skv_internal_flags_epoch();

@@ -46,28 +46,57 @@ size_t env_usize(const char *name, size_t dflt) {
     return (size_t)v;
 }
 
-// Rows below which the context is not split. The reference's default (2048,
-// src/decode_resident/utils.rs:270-278) was tuned for Apple GPUs; an explicit
-// RETI_RUST_SDPA_2PASS_MIN_LEN is honoured as is, the default here is 128 because a
-// single workgroup per kv head leaves 250 of the 256 compute units idle.
-size_t split_min_len() {
-    if (std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN")) return skv_flag_sdpa_2pass_min_len();
-    return 128;
+// Launch-shaping knobs from the environment, read once per flag generation
+// (skv_flags_reload starts a new one), not once per launch.
+struct Tuning {
+    size_t split_min_len;   // rows below which the context is not split
+    size_t target_wgs;      // workgroups a decode launch aims for
+    size_t min_pages;       // pages per split at least (0 = one per wavefront)
+    size_t forced_waves;    // 4 or 8, 0 = by shape
+    bool q_vec, fused_append, prefill_tiles;
+    size_t prefill_wgs, prefill_max_splits;
+};
+
+const Tuning &tuning() {
+    thread_local Tuning t{};
+    thread_local uint64_t seen = 0;
+    const uint64_t epoch = skv_internal_flags_epoch();
+    if (epoch != seen) {
+        // The reference's default switch-over (2048 rows, src/decode_resident/utils.rs:270-278)
+        // was tuned for Apple GPUs; an explicit RETI_RUST_SDPA_2PASS_MIN_LEN is honoured as
+        // is, the default here is 128 because a single workgroup per kv head leaves 250 of
+        // the 256 compute units idle.
+        t.split_min_len = std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN") ? skv_flag_sdpa_2pass_min_len() : 128;
+        t.target_wgs = std::max<size_t>(env_usize("SKV_DECODE_WGS", 256), 1);
+        t.min_pages = env_usize("SKV_DECODE_MIN_PAGES", 0);
+        t.forced_waves = env_usize("SKV_DECODE_WAVES", 0);
+        t.q_vec = env_usize("SKV_Q_VEC", 1) != 0;
+        t.fused_append = env_usize("SKV_FUSED_APPEND", 1) != 0;
+        t.prefill_tiles = env_usize("SKV_PREFILL_TILES", 1) != 0;
+        t.prefill_wgs = std::max<size_t>(env_usize("SKV_PREFILL_WGS", 256), 1);
+        t.prefill_max_splits = std::max<size_t>(env_usize("SKV_PREFILL_MAX_SPLITS", 512), 1);
+        seen = epoch;
+    }
+    return t;
 }
 
-// Wavefronts per workgroup of the split kernel. Eight halve the number of partials
-// for the same number of wavefronts in flight.
-int choose_waves(const skv_layer *L) {
-    const size_t w = env_usize("SKV_DECODE_WAVES", 8);
-    (void)L;
-    return w == 4 ? 4 : 8;
+// Wavefronts per workgroup of the split kernel. Eight halve the number of partials for the
+// same number of wavefronts in flight; four are better when eight would leave three
+// quarters of the compute units without a workgroup (short contexts, ring layers).
+int choose_waves(const skv_layer *L, int n_pages_scan) {
+    const size_t forced = tuning().forced_waves;
+    if (forced == 4 || forced == 8) return (int)forced;
+    const size_t kvh = (size_t)L->g.kv_heads;
+    const size_t wgs8 = kvh * std::max<size_t>(std::min<size_t>(256 / std::max<size_t>(kvh, 1), (size_t)n_pages_scan / 8), 1);
+    return wgs8 <= 64 && n_pages_scan >= 8 ? 4 : 8;
 }
 
-size_t decode_target_wgs() { return std::max<size_t>(env_usize("SKV_DECODE_WGS", 256), 1); }
+size_t decode_target_wgs() { return tuning().target_wgs; }
 
 int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows, int waves, size_t target_wgs) {
-    if (!skv_flag_sdpa_2pass_enabled() || rows < split_min_len()) return 1;
-    const size_t min_pages = std::max<size_t>(env_usize("SKV_DECODE_MIN_PAGES", (size_t)waves), 1);
+    const Tuning &t = tuning();
+    if (!skv_flag_sdpa_2pass_enabled() || rows < t.split_min_len) return 1;
+    const size_t min_pages = std::max<size_t>(t.min_pages ? t.min_pages : (size_t)waves, 1);
     size_t s = std::max<size_t>(target_wgs / (size_t)L->g.kv_heads, 1);
     s = std::min<size_t>(s, (size_t)n_pages_scan / min_pages);
     s = std::min<size_t>(s, (size_t)L->max_splits);
@@ -117,7 +146,7 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
         a.page_first = (int)(window_start / 16);
         a.n_pages = (int)((L->len + 15) / 16) - a.page_first;
     }
-    a.waves = choose_waves(L);
+    a.waves = choose_waves(L, a.n_pages);
     a.splits = choose_splits(L, a.n_pages, L->len - window_start, a.waves, target_wgs);
     // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
     // 575); log2(e) moves the softmax to base 2.
@@ -127,8 +156,7 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
     a.k_pool_w = L->k_pool;
     a.v_pool_w = L->v_pool;
     a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
-    static const bool q_vec_enabled = env_usize("SKV_Q_VEC", 1) != 0;
-    a.q_vec = (q_vec_enabled && (reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
+    a.q_vec = (tuning().q_vec && (reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
     a.g = g;
 }
 
@@ -202,17 +230,16 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     // Chunks of at least 64 query slots take the kernel that shares each K/V page among 128
     // or 256 slots through LDS; shorter ones (speculative verify rows) the decode kernel's
     // multi-query mode, one workgroup per 16 slots.
-    static const bool tiles_enabled = env_usize("SKV_PREFILL_TILES", 1) != 0;
-    const bool use_tiles = tiles_enabled && n_queries > 1 && n_queries * (size_t)g.gqa >= 64;
+    const bool use_tiles = tuning().prefill_tiles && n_queries > 1 && n_queries * (size_t)g.gqa >= 64;
     if (n_queries > 1) {
         // split the context only while the query tiles alone leave compute units idle, and
         // keep the partials in the context's scratch
         const size_t per_wg = use_tiles ? (size_t)prefill_tile_slots(g.P) : 16;
         const size_t tiles = (n_queries * (size_t)g.gqa + per_wg - 1) / per_wg * (size_t)g.kv_heads;
-        size_t want = std::max<size_t>((use_tiles ? env_usize("SKV_PREFILL_WGS", 256) : 256) / tiles, 1);
+        size_t want = std::max<size_t>((use_tiles ? tuning().prefill_wgs : 256) / tiles, 1);
         if (use_tiles) {
             want = std::min<size_t>(want, std::max<size_t>((size_t)a.n_pages / 16, 1));
-            want = std::min<size_t>(want, std::max<size_t>(env_usize("SKV_PREFILL_MAX_SPLITS", 512), 1));
+            want = std::min<size_t>(want, tuning().prefill_max_splits);
         }
         a.splits = (int)std::min<size_t>((size_t)a.splits, want);
         if (a.splits > 1) {
@@ -544,7 +571,7 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
                                float *out_dev) {
     if (!L || !k_dev || !v_dev || !q_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step: pointeur nul");
-    static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
+    const bool fused = tuning().fused_append;
     if (!fused || !uses_flash(L)) {
         int32_t rc = skv_append_device(L, stream, k_dev, k_off, v_dev, v_off);
         if (rc) return rc;
@@ -789,7 +816,7 @@ static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope,
         return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     hipStream_t s = as_stream(stream);
-    static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
+    const bool fused = tuning().fused_append;
     if (!fused || !uses_flash(L) || L->g.gqa > 16) {
         // the same step as separate launches: norm + rotation of q and k, append, attention, gate
         NormRopeArgs n{};
@@ -917,7 +944,7 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
             return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " + std::to_string(L->capacity) +
                                                " atteinte (overflow), séquence " + std::to_string(i));
     }
-    static const bool fused = env_usize("SKV_FUSED_APPEND", 1) != 0;
+    const bool fused = tuning().fused_append;
     if (!fused || !uses_flash(seqs[0]) || seqs[0]->g.gqa > 16 || n_seq == 1) {
         for (size_t i = 0; i < n_seq; ++i) {
             int32_t rc = skv_decode_step_device(seqs[i], stream, k_dev[i], 0, v_dev[i], 0, q_dev[i], out_dev[i]);
