@@ -193,6 +193,13 @@ void skv_rope_destroy(skv_rope *rope);
 int32_t skv_rms_norm_rope_decode_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
                                         size_t position, const float *x_dev, const float *weight_dev,
                                         size_t heads, size_t head_dim, float eps, float *out_dev);
+/* The same for n_rows consecutive rows (a prefill chunk): row r, contiguous after row r-1,
+ * is rotated at position_offset + r, as rms_norm_rope_heads_at does for a [seq, dim] tensor
+ * (src/decoder/attention_ops.rs:682-777, position_offset + pos at lines 736-739). */
+int32_t skv_rms_norm_rope_rows_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
+                                      size_t position_offset, const float *x_dev, const float *weight_dev,
+                                      size_t n_rows, size_t heads, size_t head_dim, float eps,
+                                      float *out_dev);
 /* DecodeResidentState::rms_norm_rope_decode (src/decode_resident/tests.rs:1168-1172, 1883):
  * host in, host out, synchronous; the rotations of `position` are computed on the host. */
 int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float *weight, size_t heads,

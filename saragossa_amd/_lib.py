@@ -89,6 +89,7 @@ SIGNATURES = {
     "skv_rope_create": (_i32, [_vp, _sz, _sz, _sz, C.c_float, C.c_float, _i32, C.POINTER(_vp)]),
     "skv_rope_destroy": (None, [_vp]),
     "skv_rms_norm_rope_decode_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _vp, _sz, _sz, C.c_float, _vp]),
+    "skv_rms_norm_rope_rows_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _sz, C.c_float, _vp]),
     "skv_rms_norm_rope_decode_host": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_float,
                                              C.c_float, C.c_float, _i32, _vp]),
     "skv_decode_step_prekv_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _sz, _vp, _vp,

@@ -194,26 +194,31 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(NormRopeArgs a) {
     __shared__ float rope[512];
     __shared__ float inv_s;
     const int head = blockIdx.x;
+    const int r = blockIdx.y; // row (position_offset + r)
     const int tid = threadIdx.x;
-    const float *x = a.x + (long)head * (a.x_head_stride > 0 ? a.x_head_stride : a.head_dim);
+    const long row_elems = (long)a.heads * a.head_dim;
+    const float *x = a.x + r * row_elems + (long)head * (a.x_head_stride > 0 ? a.x_head_stride : a.head_dim);
+    const float *rope_row = a.rope ? a.rope + (long)r * a.rope_dims : nullptr;
     for (int c = tid; c < a.head_dim; c += 256) {
         row[c] = x[c];
         w[c] = a.weight ? a.weight[c] : 1.0f;
-        rope[c] = (a.rope && c < a.rope_dims) ? a.rope[c] : 0.0f;
+        rope[c] = (rope_row && c < a.rope_dims) ? rope_row[c] : 0.0f;
     }
     __syncthreads();
     if (tid == 0) inv_s = a.weight ? head_inv_rms(row, a.head_dim, a.eps) : 1.0f;
     __syncthreads();
     const float inv = inv_s;
     for (int c = tid; c < a.head_dim; c += 256)
-        a.out[(long)head * a.head_dim + c] =
+        a.out[r * row_elems + (long)head * a.head_dim + c] =
             norm_rope_elem(row, c, inv, a.weight ? w : nullptr, a.rope ? rope : nullptr, a.rope_dims,
                            a.rope_style);
 }
 
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s) {
     if (a.heads <= 0 || a.head_dim <= 0 || a.head_dim > 512) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(norm_rope_kernel, dim3((unsigned)a.heads), dim3(256), 0, s, a);
+    const int rows = a.n_rows > 0 ? a.n_rows : 1;
+    if (rows > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(norm_rope_kernel, dim3((unsigned)a.heads, (unsigned)rows), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -763,6 +763,35 @@ int32_t skv_rms_norm_rope_decode_device(skv_ctx *ctx, skv_stream stream, const s
     return SKV_OK;
 }
 
+int32_t skv_rms_norm_rope_rows_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
+                                      size_t position_offset, const float *x_dev, const float *weight_dev,
+                                      size_t n_rows, size_t heads, size_t head_dim, float eps,
+                                      float *out_dev) {
+    if (!ctx || !x_dev || !out_dev) return fail(SKV_ERR_DEVICE, "rms_norm_rope: pointeur nul");
+    if (heads == 0 || head_dim == 0 || head_dim > 512 || heads > 65535)
+        return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE heads invalide");
+    if (n_rows == 0) return SKV_OK;
+    int32_t rc = check_rope(rope, position_offset + n_rows - 1, head_dim);
+    if (rc) return rc;
+    const size_t row_elems = heads * head_dim;
+    for (size_t first = 0; first < n_rows; first += 65535) { // grid y limit
+        const size_t n = std::min<size_t>(65535, n_rows - first);
+        NormRopeArgs a{};
+        a.x = x_dev + first * row_elems;
+        a.out = out_dev + first * row_elems;
+        a.weight = weight_dev;
+        a.rope = rope ? rope->table + (position_offset + first) * rope->rope_dims : nullptr;
+        a.heads = (int)heads;
+        a.head_dim = (int)head_dim;
+        a.rope_dims = rope ? (int)rope->rope_dims : 0;
+        a.rope_style = rope ? rope->style : 0;
+        a.eps = eps;
+        a.n_rows = (int)n;
+        SKV_HIP(launch_norm_rope(a, as_stream(stream)));
+    }
+    return SKV_OK;
+}
+
 int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float *weight, size_t heads,
                                       size_t head_dim, size_t rope_dims, size_t frequency_dim,
                                       size_t position, float eps, float theta, float position_scale,

@@ -137,6 +137,9 @@ struct NormRopeArgs {
     int heads, head_dim, rope_dims, rope_style;
     float eps;
     int x_head_stride; // elements between the heads of x (0 = head_dim)
+    // several rows at consecutive positions (grid y): row r of x and out is heads * head_dim
+    // further (contiguous rows) and uses the rotation of the position r further in the table
+    int n_rows;
 };
 
 // out[h][c] = ctx[h][c] * sigmoid(gate[h * gate_head_stride + c])

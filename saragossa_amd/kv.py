@@ -72,6 +72,13 @@ class DecodeResidentState:
                                                     _p(out)))
         return out
 
+    def encode_rms_norm_rope_rows(self, stream, rope, position_offset, x_ptr, weight_ptr, n_rows, heads,
+                                  head_dim, eps, out_ptr) -> None:
+        """rms_norm_rope_heads_at for n_rows rows at positions position_offset.. (device in/out)."""
+        check(self._l.skv_rms_norm_rope_rows_device(
+            self._h, stream, None if rope is None else rope._h, position_offset, x_ptr, weight_ptr,
+            n_rows, heads, head_dim, eps, out_ptr))
+
     def encode_attn_gate(self, stream, ctx_ptr, gate_ptr, gate_head_stride, heads, head_dim,
                          out_ptr) -> None:
         """encode_attn_gate (attn_gate_f32, src/decode_resident/kernels.rs:949-959)."""

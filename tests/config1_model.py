@@ -110,13 +110,15 @@ def norm_rope_cpu(x, heads, cfg, position):
 
 class HipKvPre(HipKv):
     """As HipKv, but a decode token hands the raw q and k projections to the library, which
-    applies the q/k norms and the rotation itself (the fused step before the cache). Prefill
-    chunks take their norm + rotation from the CPU oracle, as the other arm does."""
+    applies the q/k norms and the rotation itself (the fused step before the cache), and prefill
+    chunks go through the library's multi-row norm + rotation; the other arm takes both from
+    the CPU oracle."""
     raw_qk = True
 
     def __init__(self, cfg, capacity, state, seed=0):
         super().__init__(cfg, capacity, state, seed)
         self.cfg = cfg
+        self.state = state
         self.rope = state.rope_table(capacity, cfg.head_dim, cfg.theta)
         self.ones = torch.ones(cfg.head_dim, device="cuda")
 
@@ -129,8 +131,15 @@ class HipKvPre(HipKv):
                 v.data_ptr(), 0, self.ones.data_ptr(), self.ones.data_ptr(), cfg.eps,
                 float(cfg.head_dim), out.data_ptr())
             return out
-        q = torch.from_numpy(norm_rope_cpu(q_raw, cfg.q_heads, cfg, position)).cuda()
-        k = torch.from_numpy(norm_rope_cpu(k_raw, cfg.kv_heads, cfg, position)).cuda()
+        # a prefill chunk: the library's multi-row norm + rotation, then chunked prefill
+        q, k = torch.empty_like(q_raw), torch.empty_like(k_raw)
+        n = q_raw.shape[0]
+        self.state.encode_rms_norm_rope_rows(self.stream, self.rope, position, q_raw.data_ptr(),
+                                             self.ones.data_ptr(), n, cfg.q_heads, cfg.head_dim, cfg.eps,
+                                             q.data_ptr())
+        self.state.encode_rms_norm_rope_rows(self.stream, self.rope, position, k_raw.data_ptr(),
+                                             self.ones.data_ptr(), n, cfg.kv_heads, cfg.head_dim, cfg.eps,
+                                             k.data_ptr())
         return self.attend(li, q, k, v)
 
 
