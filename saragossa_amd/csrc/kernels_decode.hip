@@ -98,15 +98,16 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     // this lane's query slot in the B and D operand layouts
     const int my_slot = min(tile * 16 + n, n_slots - 1);
     const int my_q = MQ ? my_slot / G : 0;
-    const int my_limit = a.len - C + my_q; // last position the slot attends
-    const int my_ws = a.window > 0 ? max(a.window_start, my_limit + 1 - a.window) : a.window_start;
+    const int my_pos = a.q_pos0 + my_q;                 // position of the slot's query row
+    const int my_limit = min(my_pos, a.limit_cap);      // last position the slot attends
+    const int my_ws = a.window > 0 ? max(a.window_start, my_pos + 1 - a.window) : a.window_start;
     // extremes over the workgroup's slots
     const int qrow_lo = MQ ? (tile * 16) / G : 0;
     const int qrow_hi = MQ ? (tile * 16 + rows - 1) / G : 0;
-    const int lim_lo = a.len - C + qrow_lo;
-    const int lim_hi = a.len - C + qrow_hi;
-    const int ws_lo = a.window > 0 ? max(a.window_start, lim_lo + 1 - a.window) : a.window_start;
-    const int ws_hi = a.window > 0 ? max(a.window_start, lim_hi + 1 - a.window) : a.window_start;
+    const int lim_lo = min(a.q_pos0 + qrow_lo, a.limit_cap);
+    const int lim_hi = min(a.q_pos0 + qrow_hi, a.limit_cap);
+    const int ws_lo = a.window > 0 ? max(a.window_start, a.q_pos0 + qrow_lo + 1 - a.window) : a.window_start;
+    const int ws_hi = a.window > 0 ? max(a.window_start, a.q_pos0 + qrow_hi + 1 - a.window) : a.window_start;
 
     extern __shared__ __attribute__((aligned(16))) uint4 smem[];
     uint4 *q_hi = smem;
@@ -260,8 +261,8 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             if (tid < g.head_dim) {
                 kb = bf16_bits(k_row);
                 vb = bf16_bits(v_row);
-                a.k_pool_w[tile_at + k_index(P, r_new, tid)] = kb;
-                a.v_pool_w[tile_at + v_index(P, r_new, tid)] = vb;
+                const_cast<uint16_t *>(a.k_pool)[tile_at + k_index(P, r_new, tid)] = kb;
+                const_cast<uint16_t *>(a.v_pool)[tile_at + v_index(P, r_new, tid)] = vb;
             }
             new_k[tid] = kb;
             new_v[tid] = vb;
@@ -480,7 +481,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         if (c4 >= g.head_dim) continue;
         const int slot = tile * 16 + row;
         float *dst;
-        if (a.splits == 1) {
+        if (a.splits_total == 1) {
             acc *= 1.0f / lsum;
             if (!MQ && a.gate) {
                 const float *gp = a.gate + (long)(kvh * G + slot) * q_stride + c4;
@@ -491,7 +492,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             dst = a.out + (MQ ? ((long)(slot / G) * g.q_heads + kvh * G + slot % G)
                               : (long)(kvh * G + slot)) * g.head_dim + c4;
         } else {
-            const long pidx = ((long)kvh * a.splits + split) * n_slots + slot;
+            const long pidx = ((long)kvh * a.splits_total + a.split_base + split) * n_slots + slot;
             dst = a.part_o + pidx * g.head_dim + c4;
             if (c4 == 0) {
                 a.part_m[pidx] = mx;
@@ -500,7 +501,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         }
         if (vec_ok) {
             // partials are read once by another kernel: keep them out of the caches
-            if (a.splits == 1) *reinterpret_cast<float4_t *>(dst) = acc;
+            if (a.splits_total == 1) *reinterpret_cast<float4_t *>(dst) = acc;
             else __builtin_nontemporal_store(acc, reinterpret_cast<float4_t *>(dst));
         } else {
 #pragma unroll
@@ -548,14 +549,14 @@ __device__ __forceinline__ void decode_merge_body(const DecodeArgs &a) {
     __shared__ float red_m[16];
     __shared__ float red_l[16];
     __shared__ float acc_x[16][17];
-    const long base = ((long)kvh * a.splits) * n_slots + slot;
+    const long base = ((long)kvh * a.splits_total) * n_slots + slot;
     const long ostride = (long)n_slots * g.head_dim;
     const float *po = a.part_o + base * g.head_dim + col;
     float ov[MERGE_PER_LANE], mv[MERGE_PER_LANE], lv[MERGE_PER_LANE];
 #pragma unroll
     for (int i = 0; i < MERGE_PER_LANE; ++i) {
         const int s = sl + 16 * i;
-        const bool ok = s < a.splits;
+        const bool ok = s < a.splits_total;
         const int sc = ok ? s : 0;
         mv[i] = a.part_m[base + (long)sc * n_slots];
         lv[i] = a.part_l[base + (long)sc * n_slots];
@@ -607,7 +608,7 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
 template <int MERGE_PER_LANE>
 __global__ __launch_bounds__(256) void decode_merge_batch_kernel(DecodeBatchArgs b) {
     const DecodeArgs &a = b.seq[blockIdx.z];
-    if (a.splits <= 1) return;
+    if (a.splits_total <= 1) return;
     decode_merge_body<MERGE_PER_LANE>(a);
 }
 
@@ -650,13 +651,13 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     case 256: e = w8 ? launch_split<256, 8>(a, s) : launch_split<256, 4>(a, s); break;
     default: break;
     }
-    if (e != hipSuccess || a.splits == 1) return e;
+    if (e != hipSuccess || a.splits_total == 1) return e;
     return launch_merge(a, s);
 }
 
 hipError_t launch_merge(const DecodeArgs &a, hipStream_t s) {
     dim3 mgrid((unsigned)(a.g.kv_heads * a.n_queries * a.g.gqa), (unsigned)((a.g.head_dim + 15) / 16));
-    const int per_lane = (a.splits + 15) / 16;
+    const int per_lane = (a.splits_total + 15) / 16;
     if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_kernel<1>, mgrid, dim3(256), 0, s, a);
     else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_kernel<2>, mgrid, dim3(256), 0, s, a);
     else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_kernel<4>, mgrid, dim3(256), 0, s, a);
@@ -690,7 +691,7 @@ hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t 
     if (n_seq < 1 || n_seq > SKV_MAX_BATCH) return hipErrorInvalidValue;
     const DecodeArgs &a0 = b.seq[0];
     int max_splits = 1;
-    for (int i = 0; i < n_seq; ++i) max_splits = b.seq[i].splits > max_splits ? b.seq[i].splits : max_splits;
+    for (int i = 0; i < n_seq; ++i) max_splits = b.seq[i].splits > max_splits ? b.seq[i].splits : max_splits; // == splits_total here
     hipError_t e = hipErrorInvalidValue;
     const bool w8 = a0.waves == 8;
     switch (a0.g.P) {

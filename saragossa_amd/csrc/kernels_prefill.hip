@@ -104,11 +104,13 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
     const int wg_slot0 = blockIdx.z * (WAVES * TILES * 16);
     const int wg_slot1 = min(n_slots, wg_slot0 + WAVES * TILES * 16) - 1; // last slot of the workgroup
 
-    auto limit_of = [&](int slot) { return a.len - C + slot / G; };
-    auto ws_of = [&](int limit) { return a.window > 0 ? max(a.window_start, limit + 1 - a.window) : a.window_start; };
+    // query slot -> position of its row, last position it attends, first position it attends
+    auto pos_of = [&](int slot) { return a.q_pos0 + slot / G; };
+    auto limit_of = [&](int slot) { return min(pos_of(slot), a.limit_cap); };
+    auto ws_of = [&](int slot) { return a.window > 0 ? max(a.window_start, pos_of(slot) + 1 - a.window) : a.window_start; };
 
     // pages any slot of the workgroup can see, divided among the splits
-    const int wg_ws_lo = ws_of(limit_of(wg_slot0));
+    const int wg_ws_lo = ws_of(wg_slot0);
     const int wg_lim_hi = limit_of(wg_slot1);
     const int page_lo = g.ring_rows > 0 ? 0 : wg_ws_lo >> 4;
     const int page_hi = g.ring_rows > 0 ? a.n_pages : (wg_lim_hi >> 4) + 1;
@@ -129,11 +131,11 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
         const int s_last = min(s0 + 15, n_slots - 1);
         const int my_slot = min(s0 + n, n_slots - 1);
         my_limit[t] = limit_of(my_slot);
-        my_ws[t] = ws_of(my_limit[t]);
+        my_ws[t] = ws_of(my_slot);
         t_lim_lo[t] = limit_of(min(s0, n_slots - 1));
         t_lim_hi[t] = limit_of(s_last);
-        t_ws_lo[t] = ws_of(t_lim_lo[t]);
-        t_ws_hi[t] = ws_of(t_lim_hi[t]);
+        t_ws_lo[t] = ws_of(min(s0, n_slots - 1));
+        t_ws_hi[t] = ws_of(s_last);
         const float *qrow = a.q + ((long)(my_slot / G) * g.q_heads + kvh * G + my_slot % G) * g.head_dim;
         // eight consecutive dims of the slot's row per k-step: all loads first (two 16-byte
         // loads per step when the row allows), unconditional from clamped addresses, so that
@@ -336,11 +338,11 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
         if (!t_on[t] || slot >= n_slots) continue;
         float *dst;
         float scale = 1.0f;
-        if (a.splits == 1) {
+        if (a.splits_total == 1) {
             scale = 1.0f / l;
             dst = a.out + ((long)(slot / G) * g.q_heads + kvh * G + slot % G) * g.head_dim;
         } else {
-            const long pidx = ((long)kvh * a.splits + split) * n_slots + slot;
+            const long pidx = ((long)kvh * a.splits_total + a.split_base + split) * n_slots + slot;
             dst = a.part_o + pidx * g.head_dim;
             if (j == 0) {
                 a.part_m[pidx] = m_run[t];
@@ -377,14 +379,14 @@ __global__ __launch_bounds__(256) void merge_rows_kernel(DecodeArgs a) {
     const long ks = id / c4n;             // kvh * n_slots + slot
     const int kvh = (int)(ks / n_slots);
     const int slot = (int)(ks - (long)kvh * n_slots);
-    const long base = ((long)kvh * a.splits) * n_slots + slot;
+    const long base = ((long)kvh * a.splits_total) * n_slots + slot;
     float mx = -INFINITY;
-    for (int sp = 0; sp < a.splits; ++sp) mx = fmaxf(mx, a.part_m[base + (long)sp * n_slots]);
+    for (int sp = 0; sp < a.splits_total; ++sp) mx = fmaxf(mx, a.part_m[base + (long)sp * n_slots]);
     const float m_safe = mx == -INFINITY ? 0.0f : mx;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float lsum = 0.0f;
     const bool vec_ok = (g.head_dim & 3) == 0;
-    for (int sp = 0; sp < a.splits; ++sp) {
+    for (int sp = 0; sp < a.splits_total; ++sp) {
         const long pidx = base + (long)sp * n_slots;
         const float w = fast_exp2(a.part_m[pidx] - m_safe);
         lsum += w * a.part_l[pidx];

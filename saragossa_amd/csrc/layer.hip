@@ -4,6 +4,7 @@
 // exactly like the reference's encode-time `len += 1` (attention.rs:993).
 #include <algorithm>
 #include <cmath>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <string>
@@ -135,6 +136,9 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
     a.part_l = L->part_l;
     a.len = (int)L->len;
     a.n_queries = (int)n_queries;
+    a.q_pos0 = (int)(L->len - n_queries); // the queries are the last n_queries rows
+    a.limit_cap = INT32_MAX;
+    a.split_base = 0;
     a.window = n_queries > 1 ? (int)L->window : 0; // decode callers pass window_start themselves
     a.window_start = (int)window_start;
     if (g.ring_rows > 0) {
@@ -148,16 +152,36 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
     }
     a.waves = choose_waves(L, a.n_pages);
     a.splits = choose_splits(L, a.n_pages, L->len - window_start, a.waves, target_wgs);
+    a.splits_total = a.splits;
     // scores are multiplied by 1/sqrt(head_dim) (src/decode_resident/kernels.rs:36, 198, 395,
     // 575); log2(e) moves the softmax to base 2.
     a.qscale = (1.0f / std::sqrt((float)g.head_dim)) * 1.4426950408889634f;
     a.k_new = k_new;
     a.v_new = v_new;
-    a.k_pool_w = L->k_pool;
-    a.v_pool_w = L->v_pool;
     a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
     a.q_vec = (tuning().q_vec && (reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
     a.g = g;
+}
+
+// Split partials of a multi-query launch live in the context's scratch, grown on demand:
+// [kv_heads][n_sets][n_queries * gqa] of (o[head_dim], m, l).
+int32_t multi_query_partials(skv_layer *L, size_t n_sets, size_t n_queries, DecodeArgs &a) {
+    const Geom &g = L->g;
+    const size_t n_part = (size_t)g.kv_heads * n_sets * n_queries * g.gqa;
+    const size_t need = n_part * ((size_t)g.head_dim + 2) * sizeof(float);
+    skv_ctx *c = L->ctx;
+    if (c->mq_bytes < need) {
+        SKV_HIP(hipDeviceSynchronize());
+        if (c->mq_scratch) SKV_HIP(hipFree(c->mq_scratch));
+        c->mq_scratch = nullptr;
+        c->mq_bytes = 0;
+        SKV_HIP(hipMalloc(&c->mq_scratch, need));
+        c->mq_bytes = need;
+    }
+    a.part_o = reinterpret_cast<float *>(c->mq_scratch);
+    a.part_m = a.part_o + n_part * g.head_dim;
+    a.part_l = a.part_m + n_part;
+    return SKV_OK;
 }
 
 // k_new / v_new non-null: the row at position len-1 has not been written yet and the
@@ -242,21 +266,10 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
             want = std::min<size_t>(want, tuning().prefill_max_splits);
         }
         a.splits = (int)std::min<size_t>((size_t)a.splits, want);
+        a.splits_total = a.splits;
         if (a.splits > 1) {
-            const size_t n_part = (size_t)g.kv_heads * a.splits * n_queries * g.gqa;
-            const size_t need = n_part * ((size_t)g.head_dim + 2) * sizeof(float);
-            skv_ctx *c = L->ctx;
-            if (c->mq_bytes < need) {
-                SKV_HIP(hipDeviceSynchronize());
-                if (c->mq_scratch) SKV_HIP(hipFree(c->mq_scratch));
-                c->mq_scratch = nullptr;
-                c->mq_bytes = 0;
-                SKV_HIP(hipMalloc(&c->mq_scratch, need));
-                c->mq_bytes = need;
-            }
-            a.part_o = reinterpret_cast<float *>(c->mq_scratch);
-            a.part_m = a.part_o + n_part * g.head_dim;
-            a.part_l = a.part_m + n_part;
+            int32_t rc2 = multi_query_partials(L, (size_t)a.splits, n_queries, a);
+            if (rc2) return rc2;
         }
     }
     if (use_tiles) {
@@ -594,6 +607,58 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
     return rc;
 }
 
+// A chunk of c > 1 rows on a ring layer. The ring holds exactly the window (rounded up to a
+// page), so the chunk's own rows overwrite rows its first queries still attend. The chunk
+// is therefore attended in two phases around the append: first every query over the rows
+// already in the ring (capped at the last old position), then, once the chunk is appended,
+// over the chunk's own rows (from its first position up to each query's own). Both phases
+// leave (o, m, l) partials; one merge produces the context. c <= ring_rows.
+static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const float *k, const float *v,
+                          size_t c, float *out) {
+    const Geom &g = L->g;
+    const size_t base = L->len;
+    const size_t tiles = (c * (size_t)g.gqa + (size_t)prefill_tile_slots(g.P) - 1) / (size_t)prefill_tile_slots(g.P) *
+                         (size_t)g.kv_heads;
+    auto splits_for = [&](int n_pages) {
+        size_t want = std::max<size_t>(tuning().prefill_wgs / tiles, 1);
+        want = std::min<size_t>(want, std::max<size_t>((size_t)n_pages / 8, 1));
+        return (int)std::min<size_t>(want, tuning().prefill_max_splits);
+    };
+    DecodeArgs a1{}, a3{};
+    int s1 = 0;
+    if (base > 0) { // phase 1, prepared against the ring as it is now
+        fill_decode_args(L, q, out, L->floor_pos, nullptr, nullptr, c, tuning().prefill_wgs, a1);
+        a1.q_pos0 = (int)base;
+        a1.limit_cap = (int)base - 1;
+        s1 = splits_for(a1.n_pages);
+    }
+    const int pages_after = (int)std::min<size_t>((base + c + 15) / 16, (size_t)L->n_pages);
+    const int s3 = splits_for(pages_after);
+    const int total = s1 + s3;
+    if (base > 0) {
+        a1.splits = s1;
+        a1.split_base = 0;
+        a1.splits_total = total;
+        int32_t rc = multi_query_partials(L, (size_t)total, c, a1);
+        if (rc) return rc;
+        SKV_HIP(launch_prefill_tiles(a1, s));
+    }
+    int32_t rc = encode_append(L, s, k, v, c);
+    if (rc) return rc;
+    fill_decode_args(L, q, out, std::max(base, L->floor_pos), nullptr, nullptr, c, tuning().prefill_wgs, a3);
+    a3.q_pos0 = (int)base;
+    a3.splits = s3;
+    a3.split_base = s1;
+    a3.splits_total = total;
+    if (total > 1) {
+        rc = multi_query_partials(L, (size_t)total, c, a3);
+        if (rc) return rc;
+    }
+    SKV_HIP(launch_prefill_tiles(a3, s));
+    if (total > 1) SKV_HIP(launch_merge_rows(a3, s));
+    return SKV_OK;
+}
+
 int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q_dev,
                                  const void *k_dev, const void *v_dev, size_t n_rows,
                                  float *out_dev) {
@@ -605,19 +670,24 @@ int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q
         return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     const size_t kv_dim = skv_kv_dim(L), q_dim = (size_t)L->g.q_heads * L->g.head_dim;
-    // A ring that holds exactly its window cannot take several new rows before the first of
-    // them has been attended: the rows it would overwrite are still inside that query's
-    // window. Such layers advance in steps the ring can hold.
+    // Ring layers take the chunk in steps of at most the ring's rows (see ring_chunk).
     size_t step = std::min<size_t>(n_rows, 4096);
-    if (L->g.ring_rows > 0) {
-        const size_t room = (size_t)L->g.ring_rows >= L->window ? (size_t)L->g.ring_rows - L->window + 1 : 1;
-        step = std::min(step, room);
-    }
+    if (L->g.ring_rows > 0) step = std::min(step, (size_t)L->g.ring_rows);
     const float *q = q_dev, *k = (const float *)k_dev, *v = (const float *)v_dev;
     float *out = out_dev;
     for (size_t done = 0; done < n_rows; done += step) {
         const size_t c = std::min(step, n_rows - done);
-        int32_t rc = encode_append(L, as_stream(stream), k, v, c);
+        int32_t rc;
+        if (L->g.ring_rows > 0 && c > 1) {
+            rc = ring_chunk(L, as_stream(stream), q, k, v, c, out);
+            if (rc) return rc;
+            q += c * q_dim;
+            k += c * kv_dim;
+            v += c * kv_dim;
+            out += c * q_dim;
+            continue;
+        }
+        rc = encode_append(L, as_stream(stream), k, v, c);
         if (rc) return rc;
         const size_t ws_base = L->g.ring_rows > 0 ? L->floor_pos : 0;
         const size_t first_ws = std::max(ws_base, skv_window_start(L->len - c, L->window));

@@ -94,7 +94,11 @@ struct DecodeArgs {
     float *part_m;   // [kv_heads][splits][n_queries*gqa]   (log2 domain)
     float *part_l;   // [kv_heads][splits][n_queries*gqa]
     int len;          // rows valid: positions 0..len
-    int n_queries;    // 1 = decode; C = chunked prefill, query i attends positions <= len-C+i
+    int n_queries;    // 1 = decode; C = chunked prefill, query i sits at position q_pos0 + i
+    int q_pos0;       // position of query row 0 (len - n_queries unless the chunk is attended in two phases)
+    int limit_cap;    // no query attends beyond this position (INT_MAX = only its own causal limit)
+    int split_base;   // this launch writes partials [split_base, split_base + splits) of splits_total
+    int splits_total; // partial sets the merge will see; 1 = the launch writes the context itself
     int window;       // sliding window applied per query (0 = none)
     int window_start; // first position attended (lower bound for every query)
     int ring_base;    // ring layers: (len-1) - (len-1) % ring_rows
@@ -107,8 +111,6 @@ struct DecodeArgs {
     // fused append of the row at position len-1 (k_new null = none)
     const float *k_new; // [kv_dim] f32
     const float *v_new;
-    uint16_t *k_pool_w;
-    uint16_t *v_pool_w;
     int new_slot;     // slot that receives the row
     // fused pre-KV step (pre != 0): q and the appended k row arrive raw and get the per-head
     // RMSNorm (weights null = none) and the rotation of this position before they are used

@@ -134,3 +134,38 @@ def test_config4_sliding_window_model_batch1_and_batch4(state):
     a, _ = four[0][0][5].read_rows(ctx, 3)
     b, _ = four[1][0][5].read_rows(ctx, 3)
     assert not np.array_equal(a, b)
+
+
+def test_config4_local_layer_chunked_prefill_on_the_ring(state):
+    """BASELINE configs[4] local layer (q16/kv8/hd256, window 1024 = the ring's rows exactly):
+    a prompt prefilled in 512-row chunks equals the oracle's per-row sliding-window attention,
+    and decode continues from the ring it leaves."""
+    q_heads, kv_heads, head_dim, window = 16, 8, 256, 1024
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(44)
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r")
+    n_prompt, chunk = 1536 + 100, 512
+    kv = state.full_attention_bf16(n_prompt + 8, q_heads, kv_heads, head_dim, window=window)
+    assert kv.pages() == window // 16
+    worst = 0.0
+    for first in range(0, n_prompt, chunk):
+        c = min(chunk, n_prompt - first)
+        q = rng.standard_normal((c, q_dim), dtype=np.float32)
+        k = rng.standard_normal((c, kv_dim), dtype=np.float32)
+        v = rng.standard_normal((c, kv_dim), dtype=np.float32)
+        got = kv.prefill_rows(q, k, v)
+        want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+        worst = max(worst, float(np.abs(got - want).max()))
+    assert worst <= 1e-4, worst
+    assert kv.len() == len(cache) == n_prompt
+    gk, gv = kv.read_rows_f32(n_prompt - window, window)
+    assert np.array_equal(gk, cache.keys()[-window:]) and np.array_equal(gv, cache.values()[-window:])
+    for _ in range(4):
+        q = rng.standard_normal(q_dim, dtype=np.float32)
+        k = rng.standard_normal(kv_dim, dtype=np.float32)
+        v = rng.standard_normal(kv_dim, dtype=np.float32)
+        kv.append_row(k, v)
+        want = oracle.decode_step(cache, k, v, q, lay)
+        got = kv.attention_decode_windowed(q, skv.flags.window_start(kv.len() - 1, window))
+        assert np.abs(got - want).max() <= 1e-4
