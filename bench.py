@@ -197,6 +197,45 @@ def bench_prefill(skv, torch, np, state, stream):
     return out
 
 
+def bench_end_to_end(skv, torch, np, state):
+    """BASELINE.json configs[1] end to end: the random-init Qwen3-4B-shaped decoder of the
+    parity test (tests/config1_model.py) with its KV path on the library; 2048-token prompt in
+    512-row chunks, then greedy steps. Everything outside the KV path (embedding, projections,
+    MLP, norms, lm_head) is plain torch fp32 and only there to drive the KV path at its real
+    place in a decoder: the tok/s is dominated by those fp32 matrix products."""
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
+    from config1_model import Config, HipKvPre, Weights, forward
+    cfg = Config()
+    n_prompt, n_new, chunk = 2048, 64, 512
+    with torch.no_grad():
+        w = Weights(cfg, seed=1)
+        prompt = [int(t) for t in np.random.default_rng(1).integers(0, cfg.vocab, size=n_prompt)]
+        kv = HipKvPre(cfg, n_prompt + n_new + 8, state)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        position, logits = 0, None
+        for i in range(0, n_prompt, chunk):
+            logits = forward(cfg, w, kv, prompt[i:i + chunk], position)
+            position += chunk
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ids = []
+        for _ in range(n_new):
+            tok = int(torch.argmax(logits))
+            ids.append(tok)
+            logits = forward(cfg, w, kv, [tok], position)
+            position += 1
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+    return {"workload": "configs[1] end to end: 36 layers, 2048-token prompt in 512-row chunks, %d greedy "
+                        "steps; KV path (q/k norm + rotation, append, attention) on the library, the rest "
+                        "torch fp32" % n_new,
+            "prefill_tok_per_s": round(n_prompt / (t1 - t0), 1),
+            "decode_tok_per_s": round(n_new / (t2 - t1), 1),
+            "decode_ms_per_token": round((t2 - t1) * 1e3 / n_new, 3),
+            "distinct_ids": len(set(ids))}
+
+
 class _TimedHot:
     """HotCache with HIP events around the calls the serve path makes, so that the restore and
     snapshot legs of a turn can be told apart afterwards."""
@@ -401,6 +440,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-restore", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--end-to-end", action="store_true",
+                    help="with --config 1: also run the whole random-init decoder and report tok/s")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; every figure is one MI355X's throughput "
@@ -626,6 +667,8 @@ def main() -> int:
         result["restore"] = restore
     if recurrent is not None:
         result["recurrent_state"] = recurrent
+    if args.config == 1 and args.end_to_end:
+        result["end_to_end"] = bench_end_to_end(skv, torch, np, state)
     if args.config == 2 and not args.no_restore:
         result["prefill"] = bench_prefill(skv, torch, np, state, stream)
 
