@@ -249,6 +249,42 @@ def test_prefill_rows_equals_append_then_attention_and_causal_attention():
 
 
 # ---- RoPE + RMSNorm ----------------------------------------------------------------------
+def _golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                           "reference_known_answers.json")) as f:
+        return json.load(f)
+
+
+def test_golden_known_answers_of_the_reference():
+    """tests/golden/reference_known_answers.json: every known answer the reference's tests
+    hold for this path, as data."""
+    g = _golden()
+    for case in g["bf16_round"]["cases"]:
+        assert oracle.bf16_round(np.float32(case["input"]))[()] == np.float32(case["expected"])
+    styles = {"halves": oracle.ROPE_HALVES, "interleaved": oracle.ROPE_INTERLEAVED}
+    for case in g["apply_rope"]["cases"]:
+        got = oracle.apply_rope_heads_at([case["x"]], case["heads"], case["head_dim"], case["rope_dims"],
+                                         case["theta"], case["position"], styles[case["style"]],
+                                         position_scale=case["position_scale"],
+                                         frequency_dim=case["frequency_dim"])
+        assert np.allclose(got[0], case["expected"], atol=g["apply_rope"]["tolerance"]), case
+    t = g["two_key_attention"]
+    lay = oracle.layout(1, 1, 2, attn_scalar=t["attn_scalar"])
+    c = oracle.LayerKvCache()
+    for k, v in zip(t["keys"], t["values"]):
+        c.append([k], [v], lay)
+    out = oracle.cached_attention_one(t["query"], c, lay)
+    p0 = 1.0 / (1.0 + math.exp(-1.0 / math.sqrt(8.0)))
+    assert np.abs(out - [p0, 1 - p0]).max() <= t["tolerance"]
+    import hashlib
+    from oracle import prefix_cache as pc
+    for case in g["sha256"]["cases"]:
+        assert hashlib.sha256(case["message_utf8"].encode()).hexdigest() == case["digest_hex"]
+    assert pc.hash_for_session("abc").hex() == g["sha256"]["cases"][0]["digest_hex"]
+
+
 def test_apply_rope_styles_match_mlx_reference():
     # src/decoder/tests.rs:998-1023: constants captured from mx.fast.rope
     x = [[1.0, 2.0, 3.0, 4.0]]
