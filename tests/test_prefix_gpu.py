@@ -1,6 +1,8 @@
 """Prefix hot cache on the GPU: block snapshot / restore / gather through the hash index
 with LRU eviction, bit-exact against re-derived contents and, for the control flow,
 against the restatement of the reference's serve algorithm (src/serve/state.rs:560-639)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -60,7 +62,23 @@ def check_contents(layers, n, tokens, kv_dim):
         assert np.array_equal(gv, oracle.f32_to_bf16_bits(v)), f"layer {li} V"
 
 
-def test_snapshot_restore_roundtrip_and_clone_independence(state):
+@pytest.fixture(params=["slot-order", "layer-order"])
+def restore_order(request):
+    """Both workgroup orders of the restore copy; launches of 64 pages and more take the
+    layer order by default, the knob forces it on the small launches of these tests."""
+    if request.param == "slot-order":
+        yield request.param
+        return
+    os.environ["SKV_COPY_LAYER_MAJOR_MIN_PAGES"] = "1"
+    skv.flags.reload()
+    try:
+        yield request.param
+    finally:
+        os.environ.pop("SKV_COPY_LAYER_MAJOR_MIN_PAGES", None)
+        skv.flags.reload()
+
+
+def test_snapshot_restore_roundtrip_and_clone_independence(state, restore_order):
     # the decoder/tests.rs:297-346 pattern: restoring from a copy leaves the entry pristine
     dims, kv_dim, n = (16, 2, 256), 512, 16 * 6
     tokens = list(range(n))
@@ -144,7 +162,7 @@ class SimDecoder(pc.PromptDecoder):
 ])
 def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims, n_layers, bt,
                                                                      prefix, pool_frac,
-                                                                     chunk_blocks):
+                                                                     chunk_blocks, restore_order):
     kv_dim = dims[1] * dims[2]
     rng = np.random.default_rng(33)
     n_sessions, vocab = 6, 151936
