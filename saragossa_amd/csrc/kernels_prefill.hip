@@ -62,17 +62,32 @@ __device__ __forceinline__ void fetch_step(uint4 (&stage)[PG][(4 * (P / 32) * 32
         }
     }
 }
+// LDS order of a step: [PG/2 pairs][K tile of page A | K tile of page B | V tiles of both].
+// The K tiles are copied verbatim. The two V tiles of a pair are interleaved in 8-byte
+// halves, unit (kk, h, lane) = {page A's four keys, page B's four keys} of dim tile h, so
+// that one 16-byte read is the 32-key operand of the PV product as it stands.
 template <int P, int PG>
 __device__ __forceinline__ void store_step(const uint4 (&stage)[PG][(4 * (P / 32) * 32 + 511) / 512], uint4 *buf,
                                            int tid) {
     constexpr int TILE_U4 = (P / 32) * 64;
     constexpr int LOAD_U = (2 * TILE_U4 + 511) / 512;
+    static_assert(PG % 2 == 0, "pages are consumed in pairs");
 #pragma unroll
     for (int pg = 0; pg < PG; ++pg) {
+        uint4 *pair = buf + (pg >> 1) * 4 * TILE_U4;
 #pragma unroll
         for (int u = 0; u < LOAD_U; ++u) {
             const int i = tid + u * 512;
-            if (2 * TILE_U4 >= 512 || i < 2 * TILE_U4) buf[pg * 2 * TILE_U4 + i] = stage[pg][u];
+            if (2 * TILE_U4 < 512 && i >= 2 * TILE_U4) continue;
+            const uint4 x = stage[pg][u];
+            if (i < TILE_U4) {
+                pair[(pg & 1) * TILE_U4 + i] = x;
+            } else {
+                const int iv = i - TILE_U4;
+                uint2 *dst = reinterpret_cast<uint2 *>(pair + 2 * TILE_U4 + (iv >> 6) * 128 + (iv & 63)) + (pg & 1);
+                dst[0] = make_uint2(x.x, x.y);
+                dst[128] = make_uint2(x.z, x.w); // dim tile 1: 64 units of 16 bytes further
+            }
         }
     }
 }
@@ -213,10 +228,9 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
         const int it_a = step * PG + 2 * pp;
         if (it_a >= n_it) continue;
         const bool has_b = it_a + 1 < n_it;
-        const uint4 *kt_a = kv_lds + (step & 1) * BUF_U4 + (2 * pp) * 2 * TILE_U4;
-        const uint4 *vt_a = kt_a + TILE_U4;
-        const uint4 *kt_b = kt_a + 2 * TILE_U4;
-        const uint4 *vt_b = kt_b + TILE_U4;
+        const uint4 *kt_a = kv_lds + (step & 1) * BUF_U4 + pp * 4 * TILE_U4;
+        const uint4 *kt_b = kt_a + TILE_U4;
+        const uint4 *vt = kt_a + 2 * TILE_U4; // both pages' V tiles, interleaved (store_step)
         const int slot_a = (pb0 + it_a) * 16; // first cache slot of page A; page B follows it
 
         // which of the wavefront's tiles see the pair at all
@@ -307,14 +321,12 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
             }
         }
         // O^T += V^T . P^T over the 32 keys of the pair, the V registers shared by the tiles.
-        // Without a page B its probabilities are zero and page A's values stand in for it.
+        // Without a page B its probabilities are zero and its place holds a page the layer
+        // owns (fetch_step clamps), so the products vanish.
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-            const uint4 va = vt_a[kk * 64 + lane];
-            uint4 vb = vt_b[kk * 64 + lane];
-            if (!has_b) vb = va;
-            const bf16x8_t v0 = __builtin_bit_cast(bf16x8_t, make_uint4(va.x, va.y, vb.x, vb.y));
-            const bf16x8_t v1 = __builtin_bit_cast(bf16x8_t, make_uint4(va.z, va.w, vb.z, vb.w));
+            const bf16x8_t v0 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + lane]);
+            const bf16x8_t v1 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + 64 + lane]);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 o[t][2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, ph[t], o[t][2 * kk], 0, 0, 0);
