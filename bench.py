@@ -107,14 +107,19 @@ def bench_restore(skv, torch, np, state, stream):
     for b in range(n_tok // bt):
         h = BlockHash.chain(h, tokens[b * bt:(b + 1) * bt])
         hashes.append(h)
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    kept = hot.remember_prefix_blocks(root, hashes, bt, src, stream=stream)
-    e1.record()
-    torch.cuda.synchronize()
-    assert kept == n_tok // bt
-    snap_range_us = e0.elapsed_time(e1) * 1e3
+    samples = []
+    for _ in range(5):  # median: the first call also pays for cold code and a cold index
+        while hot.evict_lru_block() is not None:
+            pass
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        kept = hot.remember_prefix_blocks(root, hashes, bt, src, stream=stream)
+        e1.record()
+        torch.cuda.synchronize()
+        assert kept == n_tok // bt
+        samples.append(e0.elapsed_time(e1) * 1e3)
+    snap_range_us = sorted(samples)[len(samples) // 2]
     dst = make(2)
     times = []
     for it in range(13):

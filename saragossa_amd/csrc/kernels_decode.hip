@@ -18,9 +18,6 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
     return __uint_as_float(((uint32_t)b) << 16);
 }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float xor_max(float v, int mask) {
-    return fmaxf(v, __shfl_xor(v, mask, 64));
-}
 
 constexpr int DEC_MAX_SPLITS = 512;
 int decode_max_splits() { return DEC_MAX_SPLITS; }
@@ -347,8 +344,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             }
         }
         float m_blk = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
-        m_blk = xor_max(m_blk, 16);
-        m_blk = xor_max(m_blk, 32);
+        m_blk = rows_max(m_blk);
         const float m_new = fmaxf(m_run, m_blk);
         const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = fast_exp2(m_run - m_safe);
@@ -439,8 +435,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     }
 
     // this lane's share of the sum -> the query slot's sum
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = rows_sum(l_run);
 
     // ---- all wavefronts publish (o, m, l); the workgroup reduces them, four columns per thread
     __syncthreads(); // the staged queries are no longer needed: the LDS is reused

@@ -17,7 +17,6 @@ __device__ __forceinline__ uint16_t bf16_bits(float v) {
 }
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ float xor_max(float v, int mask) { return fmaxf(v, __shfl_xor(v, mask, 64)); }
 
 } // namespace
 
@@ -289,8 +288,7 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
             }
             float m_blk = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                                 fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-            m_blk = xor_max(m_blk, 16);
-            m_blk = xor_max(m_blk, 32);
+            m_blk = rows_max(m_blk);
             const float m_new = fmaxf(m_run[t], m_blk);
             const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
             const float alpha = fast_exp2(m_run[t] - m_safe);
@@ -344,8 +342,7 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
         float l = l_run[t];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        l = rows_sum(l);
         const int slot = wg_slot0 + (wave * TILES + t) * 16 + n;
         if (!t_on[t] || slot >= n_slots) continue;
         float *dst;

@@ -169,6 +169,21 @@ inline hipError_t allow_full_lds(const void *kernel, std::atomic<uint64_t> &done
 }
 
 #ifdef __HIPCC__
+// max / sum over the four 16-lane rows of a wavefront (lanes l, l^16, l^32, l^48), every
+// lane receiving the result: two row swaps in the vector unit instead of two exchanges
+// through LDS.
+__device__ __forceinline__ float rows_max(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 // sigmoid_scalar (src/decoder/attention_ops.rs:522-524)
 __device__ __forceinline__ float sigmoid_gate(float g) { return 1.0f / (1.0f + expf(-g)); }
 // The arithmetic of rms_norm_rope_heads_at (src/decoder/attention_ops.rs:682-777), operation
