@@ -345,7 +345,11 @@ int32_t skv_prefix_entry(const skv_prefix *cache, size_t index, uint8_t session[
 
 /* A pool of `pool_blocks` prefix blocks (each block_tokens/16 page slots holding K and V
  * of every layer) indexed like BlockAwarePrefixCache. `layers` fixes the shapes the pool
- * is laid out for; any set of layers with the same shapes can be used afterwards. */
+ * is laid out for; any set of layers with the same shapes can be used afterwards.
+ * Copies into and out of the pool are ordered only by the streams they are queued on: use
+ * one stream for all calls on a hot cache (the reference's server is single-threaded,
+ * src/serve/state.rs:560-646), or order the streams yourself, because an evicted block's
+ * slots are reused by the next remember without waiting for the device. */
 int32_t skv_hot_create(skv_ctx *ctx, size_t block_tokens, size_t capacity_blocks,
                        size_t blocks_per_session, size_t pool_blocks, skv_layer *const *layers,
                        size_t n_layers, skv_hot **out);

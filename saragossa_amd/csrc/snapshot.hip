@@ -309,6 +309,7 @@ int32_t skv_restore_blocks(skv_ctx *ctx, skv_stream stream, const skv_snapshot *
                            skv_layer *const *layers, size_t n_layers, const size_t *dst_block_ids,
                            size_t n_blocks) {
     if (!snap) return fail(SKV_ERR_DEVICE, "restore_blocks: snapshot nul");
+    if (n_blocks && !dst_block_ids) return fail(SKV_ERR_DEVICE, "restore_blocks: dst_block_ids nul");
     int32_t rc = check_layers(ctx, layers, n_layers);
     if (rc) return rc;
     if (!snap->sizes.empty()) return fail(SKV_ERR_DEVICE, "restore_blocks: snapshot d'état, pas de blocs");
