@@ -424,7 +424,10 @@ hipError_t launch_merge_rows(const DecodeArgs &a, hipStream_t s) {
 }
 
 // Query slots one workgroup of the kernel covers for a padded head_dim.
-int prefill_tile_slots(int P) { return P <= 64 ? 256 : 128; }
+int prefill_tile_slots(int P, bool two_tiles) { return two_tiles && prefill_two_tiles_possible(P) ? 256 : 128; }
+// Two query tiles per wavefront need twice the accumulator and query registers: up to
+// head_dim 128.
+bool prefill_two_tiles_possible(int P) { return P <= 128; }
 
 template <int P, int TILES, int PG>
 static hipError_t launch_tiles(const DecodeArgs &a, dim3 grid, hipStream_t s) {
@@ -440,12 +443,13 @@ static hipError_t launch_tiles(const DecodeArgs &a, dim3 grid, hipStream_t s) {
 
 hipError_t launch_prefill_tiles(const DecodeArgs &a, hipStream_t s) {
     const int n_slots = a.n_queries * a.g.gqa;
-    const int per_wg = prefill_tile_slots(a.g.P);
+    const bool two = a.tiles2 && prefill_two_tiles_possible(a.g.P);
+    const int per_wg = prefill_tile_slots(a.g.P, two);
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + per_wg - 1) / per_wg));
     switch (a.g.P) {
-    case 32: return launch_tiles<32, 2, 8>(a, grid, s);
-    case 64: return launch_tiles<64, 2, 8>(a, grid, s);
-    case 128: return launch_tiles<128, 1, 8>(a, grid, s);
+    case 32: return two ? launch_tiles<32, 2, 8>(a, grid, s) : launch_tiles<32, 1, 8>(a, grid, s);
+    case 64: return two ? launch_tiles<64, 2, 8>(a, grid, s) : launch_tiles<64, 1, 8>(a, grid, s);
+    case 128: return two ? launch_tiles<128, 2, 8>(a, grid, s) : launch_tiles<128, 1, 8>(a, grid, s);
     case 256: return launch_tiles<256, 1, 4>(a, grid, s);
     default: return hipErrorInvalidValue;
     }

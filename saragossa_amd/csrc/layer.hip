@@ -56,6 +56,7 @@ struct Tuning {
     size_t forced_waves;    // 4 or 8, 0 = by shape
     bool q_vec, fused_append, prefill_tiles;
     size_t prefill_wgs, prefill_max_splits;
+    long prefill_tiles2_min_pages; // -1 = by head_dim
 };
 
 const Tuning &tuning() {
@@ -76,6 +77,8 @@ const Tuning &tuning() {
         t.prefill_tiles = env_usize("SKV_PREFILL_TILES", 1) != 0;
         t.prefill_wgs = std::max<size_t>(env_usize("SKV_PREFILL_WGS", 256), 1);
         t.prefill_max_splits = std::max<size_t>(env_usize("SKV_PREFILL_MAX_SPLITS", 512), 1);
+        t.prefill_tiles2_min_pages = std::getenv("SKV_PREFILL_TILES2_MIN_PAGES")
+                                         ? (long)env_usize("SKV_PREFILL_TILES2_MIN_PAGES", 0) : -1;
         seen = epoch;
     }
     return t;
@@ -93,6 +96,18 @@ int choose_waves(const skv_layer *L, int n_pages_scan) {
 }
 
 size_t decode_target_wgs() { return tuning().target_wgs; }
+
+// Two 16-slot query tiles per wavefront in the prefill tile kernel halve the LDS reads and
+// barriers per product but also the number of workgroups. Measured with 512-row chunks: at
+// head_dim 128 they win from about 256 pages of context on (+15 % at 16k-32k rows, -4..-20 %
+// under 2k rows), at head_dim 64 from about 512 pages (+10 % at 32k rows, -10..-20 % under 4k);
+// at 256 the registers do not allow them.
+bool prefill_two_tiles(const Geom &g, int n_pages_scan) {
+    if (!prefill_two_tiles_possible(g.P)) return false;
+    const long knob = tuning().prefill_tiles2_min_pages;
+    const long min_pages = knob >= 0 ? knob : (g.P <= 64 ? 512 : 256);
+    return (long)n_pages_scan >= min_pages;
+}
 
 int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows, int waves, size_t target_wgs) {
     const Tuning &t = tuning();
@@ -258,7 +273,8 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     if (n_queries > 1) {
         // split the context only while the query tiles alone leave compute units idle, and
         // keep the partials in the context's scratch
-        const size_t per_wg = use_tiles ? (size_t)prefill_tile_slots(g.P) : 16;
+        a.tiles2 = use_tiles && prefill_two_tiles(g, a.n_pages) ? 1 : 0;
+        const size_t per_wg = use_tiles ? (size_t)prefill_tile_slots(g.P, a.tiles2 != 0) : 16;
         const size_t tiles = (n_queries * (size_t)g.gqa + per_wg - 1) / per_wg * (size_t)g.kv_heads;
         size_t want = std::max<size_t>((use_tiles ? tuning().prefill_wgs : 256) / tiles, 1);
         if (use_tiles) {
@@ -617,8 +633,9 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
                           size_t c, float *out) {
     const Geom &g = L->g;
     const size_t base = L->len;
-    const size_t tiles = (c * (size_t)g.gqa + (size_t)prefill_tile_slots(g.P) - 1) / (size_t)prefill_tile_slots(g.P) *
-                         (size_t)g.kv_heads;
+    const bool two = prefill_two_tiles(g, L->n_pages);
+    const size_t per_wg = (size_t)prefill_tile_slots(g.P, two);
+    const size_t tiles = (c * (size_t)g.gqa + per_wg - 1) / per_wg * (size_t)g.kv_heads;
     auto splits_for = [&](int n_pages) {
         size_t want = std::max<size_t>(tuning().prefill_wgs / tiles, 1);
         want = std::min<size_t>(want, std::max<size_t>((size_t)n_pages / 8, 1));
@@ -630,6 +647,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
         fill_decode_args(L, q, out, L->floor_pos, nullptr, nullptr, c, tuning().prefill_wgs, a1);
         a1.q_pos0 = (int)base;
         a1.limit_cap = (int)base - 1;
+        a1.tiles2 = two ? 1 : 0;
         s1 = splits_for(a1.n_pages);
     }
     const int pages_after = (int)std::min<size_t>((base + c + 15) / 16, (size_t)L->n_pages);
@@ -647,6 +665,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
     if (rc) return rc;
     fill_decode_args(L, q, out, std::max(base, L->floor_pos), nullptr, nullptr, c, tuning().prefill_wgs, a3);
     a3.q_pos0 = (int)base;
+    a3.tiles2 = two ? 1 : 0;
     a3.splits = s3;
     a3.split_base = s1;
     a3.splits_total = total;

@@ -126,6 +126,7 @@ struct DecodeArgs {
     const float *gate;
     int q_head_stride;
     int q_vec;              // q is 16-byte aligned and head_dim a multiple of 8: 16-byte loads
+    int tiles2;             // prefill tile kernel: two 16-slot query tiles per wavefront
     Geom g;
 };
 static_assert(sizeof(DecodeArgs) <= 256, "sixteen of them must fit the kernel argument block");
@@ -277,7 +278,8 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s);
 hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s);
 hipError_t launch_merge(const DecodeArgs &a, hipStream_t s);        // split-K partials -> context
 hipError_t launch_prefill_tiles(const DecodeArgs &a, hipStream_t s); // chunked prefill, no merge
-int prefill_tile_slots(int P);
+int prefill_tile_slots(int P, bool two_tiles);
+bool prefill_two_tiles_possible(int P);
 hipError_t launch_merge_rows(const DecodeArgs &a, hipStream_t s);    // the same merge for many query slots
 hipError_t launch_naive(const NaiveArgs &a, hipStream_t s);
 int decode_max_splits();

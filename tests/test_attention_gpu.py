@@ -194,6 +194,23 @@ def test_normal_inputs_config0(state):
 
 
 # ---- chunked prefill over the cache (multi-query, matrix cores) ----------------------------
+@pytest.fixture(params=["by-shape", "one-tile", "two-tiles"])
+def tiles_per_wavefront(request):
+    """The LDS-shared prefill kernel holds one or two 16-slot query tiles per wavefront; the
+    library picks by head_dim and context length (two only for long contexts), the knob forces
+    either so that contexts a test can afford reach both instantiations."""
+    if request.param == "by-shape":
+        yield request.param
+        return
+    os.environ["SKV_PREFILL_TILES2_MIN_PAGES"] = "0" if request.param == "two-tiles" else "1000000000"
+    skv.flags.reload()
+    try:
+        yield request.param
+    finally:
+        os.environ.pop("SKV_PREFILL_TILES2_MIN_PAGES", None)
+        skv.flags.reload()
+
+
 @pytest.mark.parametrize("dims,start,chunk,window", [
     ((32, 8, 128), 0, 64, 0),        # first chunk from an empty cache
     ((32, 8, 128), 300, 200, 0),     # later chunk, crosses page boundaries
@@ -208,7 +225,7 @@ def test_normal_inputs_config0(state):
     ((8, 1, 32), 33, 77, 0),         # head_dim 32, odd page count
     ((40, 1, 64), 10, 9, 0),         # GQA 40: 360 slots from 9 rows
 ])
-def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk, window):
+def test_prefill_rows_match_per_row_oracle(state, tiles_per_wavefront, dims, start, chunk, window):
     """One launch == the reference's per-row loop (append, then cached_attention_one)."""
     q_heads, kv_heads, head_dim = dims
     kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
@@ -238,7 +255,7 @@ def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk, window):
     (250, [7, 300, 20], (32, 2)),   # 7-row steps of 16 heads per group: the LDS-shared kernel on a ring
     (100, [130, 50], (64, 4)),
 ])
-def test_prefill_rows_on_ring_layer(state, window, chunks, heads):
+def test_prefill_rows_on_ring_layer(state, tiles_per_wavefront, window, chunks, heads):
     """A ring that holds exactly its window advances row by row; results equal the oracle's
     sliding-window attention."""
     (q_heads, kv_heads), head_dim = heads, 64
