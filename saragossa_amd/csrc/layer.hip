@@ -787,6 +787,11 @@ int32_t skv_rope_create(skv_ctx *ctx, size_t max_positions, size_t rope_dims, si
         return fail(SKV_ERR_CONFIG, "RoPE: nombre de positions invalide");
     if (rope_dims > 512) return fail(SKV_ERR_CONFIG, "RoPE: rope_dims > 512 non supporté");
     if (style != 0 && style != 1) return fail(SKV_ERR_CONFIG, "RoPE: style inconnu");
+    // one (cos, sin) pair per position and rotated pair, built on the host: keep it to a
+    // size a host vector and a device buffer always hold (1 GiB = 2 M positions at 128 dims)
+    if (max_positions * rope_dims > ((size_t)1 << 28))
+        return fail(SKV_ERR_CONFIG, "RoPE: table de " + std::to_string(max_positions) + " positions x " +
+                                        std::to_string(rope_dims) + " dims au-delà de 1 GiB");
     std::vector<float> host(max_positions * rope_dims);
     for (size_t p = 0; p < max_positions; ++p) {
         int32_t rc = skv_rope_rotations_host(p, rope_dims, frequency_dim, theta, position_scale,

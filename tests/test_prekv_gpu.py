@@ -98,6 +98,8 @@ def test_rms_norm_rope_decode_errors(state):
         state.rms_norm_rope_decode(x, w, 3, 8, 8, 0, 1e-6, 1e4)        # wrong row length
     with pytest.raises(skv.DimensionError):
         state.rms_norm_rope_decode(x, np.ones(4, np.float32), 2, 8, 8, 0, 1e-6, 1e4)
+    with pytest.raises(skv.ConfigError):
+        state.rope_table(1 << 29, 128, 1e4)      # a table no host vector should be asked for
 
 
 @pytest.fixture
