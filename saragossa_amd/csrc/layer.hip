@@ -7,6 +7,8 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -335,7 +337,7 @@ extern "C" {
 const char *skv_last_error(void) { return g_last_error.c_str(); }
 int32_t skv_abi_version(void) { return 1; }
 
-int32_t skv_ctx_create(int32_t device, skv_ctx **out) {
+int32_t skv_ctx_create(int32_t device, skv_ctx **out) try {
     if (!out) return fail(SKV_ERR_DEVICE, "skv_ctx_create: out nul");
     *out = nullptr;
     int count = 0;
@@ -354,6 +356,8 @@ int32_t skv_ctx_create(int32_t device, skv_ctx **out) {
     c->stream = nullptr;
     *out = c;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 void skv_ctx_destroy(skv_ctx *ctx) {
@@ -364,11 +368,13 @@ void skv_ctx_destroy(skv_ctx *ctx) {
     delete ctx;
 }
 
-int32_t skv_ctx_synchronize(skv_ctx *ctx) {
+int32_t skv_ctx_synchronize(skv_ctx *ctx) try {
     if (!ctx) return fail(SKV_ERR_DEVICE, "ctx nul");
     SKV_HIP(hipSetDevice(ctx->device));
     SKV_HIP(hipDeviceSynchronize());
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 void skv_layer_destroy(skv_layer *L) {
@@ -383,7 +389,7 @@ void skv_layer_destroy(skv_layer *L) {
 }
 
 int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
-                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) {
+                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) try {
     if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_layer_create: pointeur nul");
     *out = nullptr;
     if (capacity == 0 || q_heads == 0 || kv_heads == 0 || head_dim == 0)
@@ -453,15 +459,19 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     }
     *out = L;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_layer_create_for(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
-                             size_t head_dim, int32_t sampled, skv_layer **out) {
+                             size_t head_dim, int32_t sampled, skv_layer **out) try {
     const int32_t dtype = skv_flag_kv_bf16_for(sampled) ? SKV_DTYPE_BF16 : SKV_DTYPE_F32;
     return skv_layer_create(ctx, capacity, q_heads, kv_heads, head_dim, dtype, 0, out);
+} catch (...) {
+    return skv::fail_exception();
 }
 
-int32_t skv_layer_set_block_table(skv_layer *L, const int32_t *table, size_t n) {
+int32_t skv_layer_set_block_table(skv_layer *L, const int32_t *table, size_t n) try {
     if (!L || !table) return fail(SKV_ERR_DEVICE, "set_block_table: pointeur nul");
     if (L->len != 0) return fail(SKV_ERR_DIMENSION, "set_block_table: cache non vide");
     if (n != (size_t)L->n_pages)
@@ -479,6 +489,8 @@ int32_t skv_layer_set_block_table(skv_layer *L, const int32_t *table, size_t n) 
                            L->ctx->stream));
     SKV_HIP(hipStreamSynchronize(L->ctx->stream));
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 size_t skv_layer_pages(const skv_layer *L) { return L ? (size_t)L->n_pages : 0; }
@@ -493,7 +505,7 @@ size_t skv_logical_byte_len(const skv_layer *L) {
     return L ? L->capacity * (size_t)L->g.kv_heads * L->g.head_dim * 2 : 0;
 }
 
-int32_t skv_truncate(skv_layer *L, size_t len) {
+int32_t skv_truncate(skv_layer *L, size_t len) try {
     if (!L) return fail(SKV_ERR_DEVICE, "truncate: pointeur nul");
     if (len > L->capacity)
         return fail(SKV_ERR_DIMENSION, "truncate KV " + std::to_string(len) + " > capacité " +
@@ -501,10 +513,12 @@ int32_t skv_truncate(skv_layer *L, size_t len) {
     L->len = len;
     if (len == 0) L->floor_pos = 0;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_seed(skv_layer *L, const float *keys, const float *values, size_t n_elems,
-                 size_t n_rows) {
+                 size_t n_rows) try {
     if (!L) return fail(SKV_ERR_DEVICE, "seed: pointeur nul");
     if (n_rows > L->capacity)
         return fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(n_rows) + " > capacité " +
@@ -534,9 +548,11 @@ int32_t skv_seed(skv_layer *L, const float *keys, const float *values, size_t n_
     if (rc) return rc;
     if (e2 != hipSuccess) return fail_hip(e2, "seed: synchronisation");
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
-int32_t skv_append_host(skv_layer *L, const float *key, const float *value, size_t n_elems) {
+int32_t skv_append_host(skv_layer *L, const float *key, const float *value, size_t n_elems) try {
     if (!L || !key || !value) return fail(SKV_ERR_DEVICE, "append: pointeur nul");
     const size_t kv_dim = skv_kv_dim(L);
     if (n_elems != kv_dim)
@@ -553,32 +569,40 @@ int32_t skv_append_host(skv_layer *L, const float *key, const float *value, size
     if (rc) return rc;
     SKV_HIP(hipStreamSynchronize(s));
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_append_device(skv_layer *L, skv_stream stream, const void *k_dev, size_t k_off,
-                          const void *v_dev, size_t v_off) {
+                          const void *v_dev, size_t v_off) try {
     if (!L || !k_dev || !v_dev) return fail(SKV_ERR_DEVICE, "append device: pointeur nul");
     if ((k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "append device: offset non aligné f32");
     return encode_append(L, as_stream(stream),
                          reinterpret_cast<const float *>((const char *)k_dev + k_off),
                          reinterpret_cast<const float *>((const char *)v_dev + v_off), 1);
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_append_batch_device(skv_layer *L, skv_stream stream, const void *k_dev,
-                                const void *v_dev, size_t n_rows) {
+                                const void *v_dev, size_t n_rows) try {
     if (!L || !k_dev || !v_dev) return fail(SKV_ERR_DEVICE, "append batch: pointeur nul");
     if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "cache KV batch attend seq > 0");
     return encode_append(L, as_stream(stream), (const float *)k_dev, (const float *)v_dev, n_rows);
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_attention_device(skv_layer *L, skv_stream stream, const float *q_dev, float *out_dev,
-                             size_t window_start) {
+                             size_t window_start) try {
     if (!L || !q_dev || !out_dev) return fail(SKV_ERR_DEVICE, "attention device: pointeur nul");
     return encode_attention(L, as_stream(stream), q_dev, out_dev, window_start);
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_attention_host(skv_layer *L, const float *q, size_t n_elems, size_t window_start,
-                           float *out) {
+                           float *out) try {
     if (!L || !q || !out) return fail(SKV_ERR_DEVICE, "attention: pointeur nul");
     if (L->len == 0) return fail(SKV_ERR_DIMENSION, "attention_decode sur KV vide");
     const size_t q_dim = (size_t)L->g.q_heads * L->g.head_dim;
@@ -593,11 +617,13 @@ int32_t skv_attention_host(skv_layer *L, const float *q, size_t n_elems, size_t 
     SKV_HIP(hipMemcpyAsync(out, L->out_stage, q_dim * sizeof(float), hipMemcpyDeviceToHost, s));
     SKV_HIP(hipStreamSynchronize(s));
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_dev, size_t k_off,
                                const void *v_dev, size_t v_off, const float *q_dev,
-                               float *out_dev) {
+                               float *out_dev) try {
     if (!L || !k_dev || !v_dev || !q_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step: pointeur nul");
     const bool fused = tuning().fused_append;
@@ -621,6 +647,8 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
                                   reinterpret_cast<const float *>((const char *)v_dev + v_off));
     if (rc) L->len -= 1;
     return rc;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 // A chunk of c > 1 rows on a ring layer. The ring holds exactly the window (rounded up to a
@@ -680,7 +708,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
 
 int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q_dev,
                                  const void *k_dev, const void *v_dev, size_t n_rows,
-                                 float *out_dev) {
+                                 float *out_dev) try {
     if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "prefill chunk: pointeur nul");
     if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "attention batch cached shapes: seq == 0");
@@ -722,10 +750,12 @@ int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q
         out += c * q_dim;
     }
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_prefill_chunk_host(skv_layer *L, const float *q, const float *k, const float *v,
-                               size_t n_rows, float *out) {
+                               size_t n_rows, float *out) try {
     if (!L || !q || !k || !v || !out) return fail(SKV_ERR_DEVICE, "prefill chunk: pointeur nul");
     if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "attention batch cached shapes: seq == 0");
     SKV_HIP(hipSetDevice(L->ctx->device));
@@ -748,6 +778,8 @@ int32_t skv_prefill_chunk_host(skv_layer *L, const float *q, const float *k, con
     if (rc) return rc;
     if (e2 != hipSuccess) return fail_hip(e2, "prefill chunk: synchronisation");
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 // ---- the step before the cache: per-head RMSNorm + rotation --------------------------
@@ -761,7 +793,7 @@ struct skv_rope {
 };
 
 int32_t skv_rope_rotations_host(size_t position, size_t rope_dims, size_t frequency_dim, float theta,
-                                float position_scale, float *cos_sin_out) {
+                                float position_scale, float *cos_sin_out) try {
     if (!cos_sin_out) return fail(SKV_ERR_DEVICE, "rope: pointeur nul");
     if (rope_dims == 0 || rope_dims % 2 != 0)
         return fail(SKV_ERR_DIMENSION, "RoPE: rope_dims=" + std::to_string(rope_dims) + " doit être pair et non nul");
@@ -777,10 +809,12 @@ int32_t skv_rope_rotations_host(size_t position, size_t rope_dims, size_t freque
         cos_sin_out[2 * pair + 1] = sinf(angle);
     }
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_rope_create(skv_ctx *ctx, size_t max_positions, size_t rope_dims, size_t frequency_dim,
-                        float theta, float position_scale, int32_t style, skv_rope **out) {
+                        float theta, float position_scale, int32_t style, skv_rope **out) try {
     if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_rope_create: pointeur nul");
     *out = nullptr;
     if (max_positions == 0 || max_positions > ((size_t)1 << 30))
@@ -814,6 +848,8 @@ int32_t skv_rope_create(skv_ctx *ctx, size_t max_positions, size_t rope_dims, si
     }
     *out = r;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 void skv_rope_destroy(skv_rope *rope) {
@@ -837,7 +873,7 @@ static int32_t check_rope(const skv_rope *rope, size_t position, size_t head_dim
 
 int32_t skv_rms_norm_rope_decode_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
                                         size_t position, const float *x_dev, const float *weight_dev,
-                                        size_t heads, size_t head_dim, float eps, float *out_dev) {
+                                        size_t heads, size_t head_dim, float eps, float *out_dev) try {
     if (!ctx || !x_dev || !out_dev) return fail(SKV_ERR_DEVICE, "rms_norm_rope: pointeur nul");
     if (heads == 0 || head_dim == 0 || head_dim > 512 || heads > 65535)
         return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE heads invalide");
@@ -855,12 +891,14 @@ int32_t skv_rms_norm_rope_decode_device(skv_ctx *ctx, skv_stream stream, const s
     a.eps = eps;
     SKV_HIP(launch_norm_rope(a, as_stream(stream)));
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_rms_norm_rope_rows_device(skv_ctx *ctx, skv_stream stream, const skv_rope *rope,
                                       size_t position_offset, const float *x_dev, const float *weight_dev,
                                       size_t n_rows, size_t heads, size_t head_dim, float eps,
-                                      float *out_dev) {
+                                      float *out_dev) try {
     if (!ctx || !x_dev || !out_dev) return fail(SKV_ERR_DEVICE, "rms_norm_rope: pointeur nul");
     if (heads == 0 || head_dim == 0 || head_dim > 512 || heads > 65535)
         return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE heads invalide");
@@ -884,12 +922,14 @@ int32_t skv_rms_norm_rope_rows_device(skv_ctx *ctx, skv_stream stream, const skv
         SKV_HIP(launch_norm_rope(a, as_stream(stream)));
     }
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float *weight, size_t heads,
                                       size_t head_dim, size_t rope_dims, size_t frequency_dim,
                                       size_t position, float eps, float theta, float position_scale,
-                                      int32_t style, float *out) {
+                                      int32_t style, float *out) try {
     if (!ctx || !x || !out) return fail(SKV_ERR_DEVICE, "rms_norm_rope: pointeur nul");
     if (heads == 0 || head_dim == 0 || head_dim > 512 || heads > 65535)
         return fail(SKV_ERR_DIMENSION, "RMSNorm/RoPE heads invalide");
@@ -925,6 +965,8 @@ int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float 
     if (e != hipSuccess) return fail_hip(e, "rms_norm_rope");
     if (e2 != hipSuccess) return fail_hip(e2, "rms_norm_rope: synchronisation");
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope, size_t position,
@@ -997,7 +1039,7 @@ int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_
                                      size_t position, const void *q_dev, size_t q_off,
                                      const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
                                      const float *q_norm_w, const float *k_norm_w, float eps,
-                                     float attn_scalar, float *out_dev) {
+                                     float attn_scalar, float *out_dev) try {
     if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step_prekv: pointeur nul");
     if ((q_off | k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "decode_step_prekv: offset non aligné f32");
@@ -1006,13 +1048,15 @@ int32_t skv_decode_step_prekv_device(skv_layer *L, skv_stream stream, const skv_
                       reinterpret_cast<const float *>((const char *)k_dev + k_off),
                       reinterpret_cast<const float *>((const char *)v_dev + v_off), q_norm_w,
                       k_norm_w, eps, attn_scalar, out_dev);
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_decode_step_gated_device(skv_layer *L, skv_stream stream, const skv_rope *rope,
                                      size_t position, const void *qg_dev, size_t qg_off,
                                      const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,
                                      const float *q_norm_w, const float *k_norm_w, float eps,
-                                     float attn_scalar, float *out_dev) {
+                                     float attn_scalar, float *out_dev) try {
     if (!L || !qg_dev || !k_dev || !v_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step_gated: pointeur nul");
     if ((qg_off | k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "decode_step_gated: offset non aligné f32");
@@ -1024,10 +1068,12 @@ int32_t skv_decode_step_gated_device(skv_layer *L, skv_stream stream, const skv_
                       reinterpret_cast<const float *>((const char *)k_dev + k_off),
                       reinterpret_cast<const float *>((const char *)v_dev + v_off), q_norm_w,
                       k_norm_w, eps, attn_scalar, out_dev);
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_attn_gate_device(skv_ctx *ctx, skv_stream stream, const float *ctx_dev, const float *gate_dev,
-                             size_t gate_head_stride, size_t heads, size_t head_dim, float *out_dev) {
+                             size_t gate_head_stride, size_t heads, size_t head_dim, float *out_dev) try {
     if (!ctx || !ctx_dev || !gate_dev || !out_dev) return fail(SKV_ERR_DEVICE, "attn_gate: pointeur nul");
     if (heads == 0 || head_dim == 0 || heads * head_dim > ((size_t)1 << 30))
         return fail(SKV_ERR_DIMENSION, "attn_gate: dimensions invalides");
@@ -1042,11 +1088,13 @@ int32_t skv_attn_gate_device(skv_ctx *ctx, skv_stream stream, const float *ctx_d
     ga.gate_head_stride = (int)(gate_head_stride ? gate_head_stride : head_dim);
     SKV_HIP(launch_gate(ga, as_stream(stream)));
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_stream stream,
                                      const void *const *k_dev, const void *const *v_dev,
-                                     const float *const *q_dev, float *const *out_dev) {
+                                     const float *const *q_dev, float *const *out_dev) try {
     if (!seqs || !k_dev || !v_dev || !q_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step_batch: pointeur nul");
     if (n_seq == 0) return fail(SKV_ERR_DIMENSION, "decode_step_batch: aucune séquence");
@@ -1107,11 +1155,13 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
         }
     }
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_decode_step_layers_device(skv_layer *const *layers, size_t n_layers, skv_stream stream,
                                       const void *const *k_dev, const void *const *v_dev,
-                                      const float *const *q_dev, float *const *out_dev) {
+                                      const float *const *q_dev, float *const *out_dev) try {
     if (!layers || !k_dev || !v_dev || !q_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step_layers: pointeur nul");
     for (size_t i = 0; i < n_layers; ++i) {
@@ -1120,6 +1170,8 @@ int32_t skv_decode_step_layers_device(skv_layer *const *layers, size_t n_layers,
         if (rc) return rc;
     }
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 static int32_t check_rows(const skv_layer *L, size_t first, size_t n) {
@@ -1134,7 +1186,7 @@ static int32_t check_rows(const skv_layer *L, size_t first, size_t n) {
 }
 
 int32_t skv_gather_device(skv_layer *L, skv_stream stream, size_t first, size_t n, void *k_dst,
-                          void *v_dst) {
+                          void *v_dst) try {
     if (!L) return fail(SKV_ERR_DEVICE, "gather: pointeur nul");
     int32_t rc = check_rows(L, first, n);
     if (rc) return rc;
@@ -1150,9 +1202,11 @@ int32_t skv_gather_device(skv_layer *L, skv_stream stream, size_t first, size_t 
     a.g = L->g;
     SKV_HIP(launch_gather(a, as_stream(stream)));
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
-int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uint16_t *v_out) {
+int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uint16_t *v_out) try {
     if (!L) return fail(SKV_ERR_DEVICE, "read_rows: pointeur nul");
     int32_t rc = check_rows(L, first, n);
     if (rc) return rc;
@@ -1173,6 +1227,8 @@ int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uin
     if (e != hipSuccess) return fail_hip(e, "read_rows: copie device→hôte");
     if (e2 != hipSuccess) return fail_hip(e2, "read_rows: synchronisation");
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 } // extern "C"

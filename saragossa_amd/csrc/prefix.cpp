@@ -391,15 +391,19 @@ void skv_hash_chain(const uint8_t previous[32], const uint64_t *tokens, size_t n
 }
 
 int32_t skv_prefix_create(size_t block_tokens, size_t capacity, size_t blocks_per_session,
-                          skv_prefix **out) {
+                          skv_prefix **out) try {
     if (!out) return fail(SKV_ERR_DEVICE, "skv_prefix_create: out nul");
     *out = new skv_prefix(block_tokens, capacity, blocks_per_session);
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
-int32_t skv_prefix_from_runtime_flags(skv_prefix **out) {
+int32_t skv_prefix_from_runtime_flags(skv_prefix **out) try {
     return skv_prefix_create(skv_flag_serve_prefix_block_tokens(), skv_flag_serve_prefix_cache_blocks(),
                              skv_flag_serve_prefix_blocks_per_session(), out);
+} catch (...) {
+    return skv::fail_exception();
 }
 
 void skv_prefix_destroy(skv_prefix *cache) { delete cache; }
@@ -413,7 +417,7 @@ size_t skv_prefix_session_block_count(const skv_prefix *c, const uint8_t session
 }
 
 int32_t skv_prefix_match(skv_prefix *c, const uint8_t root[32], const uint64_t *tokens, size_t n,
-                         int32_t *found, skv_hit *hit, uint64_t *chain_payloads, size_t chain_cap) {
+                         int32_t *found, skv_hit *hit, uint64_t *chain_payloads, size_t chain_cap) try {
     if (!c || !root || !found || (n && !tokens)) return fail(SKV_ERR_DEVICE, "prefix_match: pointeur nul");
     PrefixHit h{};
     std::vector<uint64_t> chain;
@@ -428,11 +432,13 @@ int32_t skv_prefix_match(skv_prefix *c, const uint8_t root[32], const uint64_t *
     if (chain_payloads)
         for (size_t i = 0; i < chain.size() && i < chain_cap; ++i) chain_payloads[i] = chain[i];
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_prefix_insert(skv_prefix *c, const uint8_t session[32], const uint8_t hash[32],
                           size_t tokens, uint64_t payload, size_t bytes, uint64_t *dropped,
-                          size_t dropped_cap, size_t *n_dropped, size_t *bytes_out) {
+                          size_t dropped_cap, size_t *n_dropped, size_t *bytes_out) try {
     if (!c || !session || !hash) return fail(SKV_ERR_DEVICE, "prefix_insert: pointeur nul");
     if (dropped && dropped_cap < 4)
         return fail(SKV_ERR_DIMENSION, "prefix_insert: dropped doit offrir au moins 4 places");
@@ -443,20 +449,26 @@ int32_t skv_prefix_insert(skv_prefix *c, const uint8_t session[32], const uint8_
     if (n_dropped) *n_dropped = gone.size();
     if (bytes_out) *bytes_out = b;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
-int32_t skv_prefix_evict_lru(skv_prefix *c, int32_t *found, uint64_t *payload, size_t *bytes) {
+int32_t skv_prefix_evict_lru(skv_prefix *c, int32_t *found, uint64_t *payload, size_t *bytes) try {
     if (!c || !found) return fail(SKV_ERR_DEVICE, "prefix_evict_lru: pointeur nul");
     *found = c->index.evict_lru(payload, bytes) ? 1 : 0;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_prefix_entry(const skv_prefix *c, size_t index, uint8_t session[32], uint8_t hash[32],
-                         size_t *tokens, uint64_t *payload, size_t *bytes) {
+                         size_t *tokens, uint64_t *payload, size_t *bytes) try {
     if (!c) return fail(SKV_ERR_DEVICE, "prefix_entry: pointeur nul");
     if (!c->index.entry(index, session, hash, tokens, payload, bytes))
         return fail(SKV_ERR_DIMENSION, "prefix_entry: index " + std::to_string(index) + " hors plage");
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 } // extern "C"

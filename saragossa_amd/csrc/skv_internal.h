@@ -6,6 +6,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <exception>
+#include <new>
 #include <string>
 
 #include "../../include/saragossa_kv.h"
@@ -15,6 +17,20 @@ namespace skv {
 // ---- errors -------------------------------------------------------------------
 void set_error(const std::string &msg);
 int32_t fail(int32_t code, const std::string &msg);
+// Called from the catch-all of an entry point: the exception in flight becomes a status code
+// and a message (nothing C++ crosses the C boundary; the reference never panics on a
+// fallible path either).
+inline int32_t fail_exception() {
+    try {
+        throw;
+    } catch (const std::bad_alloc &) {
+        return fail(SKV_ERR_DEVICE, "mémoire hôte épuisée");
+    } catch (const std::exception &e) {
+        return fail(SKV_ERR_DEVICE, std::string("exception: ") + e.what());
+    } catch (...) {
+        return fail(SKV_ERR_DEVICE, "exception inconnue");
+    }
+}
 int32_t fail_hip(hipError_t e, const char *what);
 
 #define SKV_HIP(expr)                                            \

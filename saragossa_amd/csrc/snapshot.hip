@@ -263,7 +263,7 @@ extern "C" {
 // ---- block snapshots ----------------------------------------------------------------------
 int32_t skv_snapshot_blocks(skv_ctx *ctx, skv_stream stream, skv_layer *const *layers,
                             size_t n_layers, const size_t *block_ids, size_t n_blocks,
-                            skv_snapshot **out) {
+                            skv_snapshot **out) try {
     if (!out) return fail(SKV_ERR_DEVICE, "snapshot_blocks: out nul");
     *out = nullptr;
     int32_t rc = check_layers(ctx, layers, n_layers);
@@ -303,11 +303,13 @@ int32_t skv_snapshot_blocks(skv_ctx *ctx, skv_stream stream, skv_layer *const *l
     }
     *out = snap;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_restore_blocks(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snap,
                            skv_layer *const *layers, size_t n_layers, const size_t *dst_block_ids,
-                           size_t n_blocks) {
+                           size_t n_blocks) try {
     if (!snap) return fail(SKV_ERR_DEVICE, "restore_blocks: snapshot nul");
     if (n_blocks && !dst_block_ids) return fail(SKV_ERR_DEVICE, "restore_blocks: dst_block_ids nul");
     int32_t rc = check_layers(ctx, layers, n_layers);
@@ -335,10 +337,12 @@ int32_t skv_restore_blocks(skv_ctx *ctx, skv_stream stream, const skv_snapshot *
     SKV_HIP(hipSetDevice(ctx->device));
     return copy_pages(snap->layout, snap->base, layers, n_layers, pages.data(), slots.data(), n_blocks,
                       nullptr, false, as_stream(stream));
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_snapshot_clone(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snap,
-                           skv_snapshot **out) {
+                           skv_snapshot **out) try {
     if (!ctx || !snap || !out) return fail(SKV_ERR_DEVICE, "snapshot_clone: pointeur nul");
     *out = nullptr;
     SKV_HIP(hipSetDevice(ctx->device));
@@ -360,6 +364,8 @@ int32_t skv_snapshot_clone(skv_ctx *ctx, skv_stream stream, const skv_snapshot *
     }
     *out = c;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 size_t skv_snapshot_bytes(const skv_snapshot *snap) { return snap ? snap->bytes : 0; }
@@ -376,7 +382,7 @@ void skv_snapshot_free(skv_snapshot *snap) {
 
 // ---- recurrent-state snapshots ---------------------------------------------------------------
 int32_t skv_state_snapshot(skv_ctx *ctx, skv_stream stream, const void *const *dev_ptrs,
-                           const size_t *bytes, size_t n, skv_snapshot **out) {
+                           const size_t *bytes, size_t n, skv_snapshot **out) try {
     if (!ctx || !out || (n && (!dev_ptrs || !bytes))) return fail(SKV_ERR_DEVICE, "state_snapshot: pointeur nul");
     *out = nullptr;
     SKV_HIP(hipSetDevice(ctx->device));
@@ -410,10 +416,12 @@ int32_t skv_state_snapshot(skv_ctx *ctx, skv_stream stream, const void *const *d
     if (n == 0) snap->sizes.clear();
     *out = snap;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 int32_t skv_state_restore(skv_ctx *ctx, skv_stream stream, const skv_snapshot *snap,
-                          void *const *dev_ptrs, const size_t *bytes, size_t n) {
+                          void *const *dev_ptrs, const size_t *bytes, size_t n) try {
     if (!ctx || !snap || (n && (!dev_ptrs || !bytes))) return fail(SKV_ERR_DEVICE, "state_restore: pointeur nul");
     if (n != snap->sizes.size())
         return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=" + std::to_string(snap->sizes.size()) +
@@ -426,12 +434,14 @@ int32_t skv_state_restore(skv_ctx *ctx, skv_stream stream, const skv_snapshot *s
     std::vector<const void *> src(n);
     for (size_t i = 0; i < n; ++i) src[i] = snap->base + snap->offsets[i];
     return launch_flat(src.data(), dev_ptrs, bytes, n, as_stream(stream));
+} catch (...) {
+    return skv::fail_exception();
 }
 
 // ---- the hot cache: page pool + index ----------------------------------------------------------
 int32_t skv_hot_create(skv_ctx *ctx, size_t block_tokens, size_t capacity_blocks,
                        size_t blocks_per_session, size_t pool_blocks, skv_layer *const *layers,
-                       size_t n_layers, skv_hot **out) {
+                       size_t n_layers, skv_hot **out) try {
     if (!out) return fail(SKV_ERR_DEVICE, "hot_create: out nul");
     *out = nullptr;
     int32_t rc = check_layers(ctx, layers, n_layers);
@@ -458,6 +468,8 @@ int32_t skv_hot_create(skv_ctx *ctx, size_t block_tokens, size_t capacity_blocks
     for (size_t i = h->pool_slots; i-- > 0;) h->free_slots.push_back((int32_t)i);
     *out = h;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 void skv_hot_destroy(skv_hot *h) {
@@ -481,14 +493,16 @@ uint64_t skv_hot_evictions(const skv_hot *h) { return h ? h->evictions : 0; }
 uint64_t skv_hot_skipped(const skv_hot *h) { return h ? h->skipped : 0; }
 
 int32_t skv_hot_entry(const skv_hot *h, size_t index, uint8_t session[32], uint8_t hash[32],
-                      size_t *tokens, size_t *bytes) {
+                      size_t *tokens, size_t *bytes) try {
     if (!h) return fail(SKV_ERR_DEVICE, "hot_entry: pointeur nul");
     if (!h->index->entry(index, session, hash, tokens, nullptr, bytes))
         return fail(SKV_ERR_DIMENSION, "hot_entry: index " + std::to_string(index) + " hors plage");
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
-int32_t skv_hot_evict_lru(skv_hot *h, int32_t *found, size_t *bytes) {
+int32_t skv_hot_evict_lru(skv_hot *h, int32_t *found, size_t *bytes) try {
     if (!h || !found) return fail(SKV_ERR_DEVICE, "hot_evict_lru: pointeur nul");
     uint64_t id = 0;
     const bool ok = h->index->evict_lru(&id, bytes);
@@ -498,6 +512,8 @@ int32_t skv_hot_evict_lru(skv_hot *h, int32_t *found, size_t *bytes) {
         ++h->evictions;
     }
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 // remember_prefix_block (src/serve/state.rs:613-639): snapshot the block that ends at
@@ -506,7 +522,7 @@ int32_t skv_hot_evict_lru(skv_hot *h, int32_t *found, size_t *bytes) {
 int32_t skv_hot_remember(skv_hot *h, skv_stream stream, const uint8_t session[32],
                          const uint8_t hash[32], size_t tokens, skv_layer *const *layers,
                          size_t n_layers, const void *const *state_ptrs, const size_t *state_bytes,
-                         size_t n_states, int32_t *cached) {
+                         size_t n_states, int32_t *cached) try {
     if (!h || !session || !hash || !cached) return fail(SKV_ERR_DEVICE, "hot_remember: pointeur nul");
     *cached = 0;
     int32_t rc = check_layers(h->ctx, layers, n_layers);
@@ -561,6 +577,8 @@ int32_t skv_hot_remember(skv_hot *h, skv_stream stream, const uint8_t session[32
     }
     *cached = h->entries.count(id) ? 1 : 0;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 // remember_prefix_block for `n_blocks` consecutive boundaries in one call: block i covers
@@ -570,7 +588,7 @@ int32_t skv_hot_remember(skv_hot *h, skv_stream stream, const uint8_t session[32
 // state (a state exists only at the boundary the decoder is at).
 int32_t skv_hot_remember_range(skv_hot *h, skv_stream stream, const uint8_t session[32],
                                const uint8_t *hashes, size_t first_tokens, size_t n_blocks,
-                               skv_layer *const *layers, size_t n_layers, size_t *n_cached) {
+                               skv_layer *const *layers, size_t n_layers, size_t *n_cached) try {
     if (!h || !session || (n_blocks && !hashes)) return fail(SKV_ERR_DEVICE, "hot_remember_range: pointeur nul");
     if (n_cached) *n_cached = 0;
     int32_t rc = check_layers(h->ctx, layers, n_layers);
@@ -650,6 +668,8 @@ int32_t skv_hot_remember_range(skv_hot *h, skv_stream stream, const uint8_t sess
     if (rc) return rc;
     if (n_cached) *n_cached = cached;
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 // The hit branch of prefill_prompt_state (src/serve/state.rs:574-584): longest chain of
@@ -658,7 +678,7 @@ int32_t skv_hot_remember_range(skv_hot *h, skv_stream stream, const uint8_t sess
 int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[32],
                               const uint64_t *tokens, size_t n_tokens, skv_layer *const *layers,
                               size_t n_layers, void *const *state_ptrs, const size_t *state_bytes,
-                              size_t n_states, size_t *reused_tokens, uint8_t hash_out[32]) {
+                              size_t n_states, size_t *reused_tokens, uint8_t hash_out[32]) try {
     if (!h || !root || !reused_tokens || (n_tokens && !tokens))
         return fail(SKV_ERR_DEVICE, "hot_match_restore: pointeur nul");
     *reused_tokens = 0;
@@ -745,6 +765,8 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
     *reused_tokens = reused;
     if (hash_out) std::memcpy(hash_out, hit.hash, 32);
     return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
 }
 
 } // extern "C"
