@@ -621,8 +621,16 @@ int32_t skv_hot_remember_range(skv_hot *h, skv_stream stream, const uint8_t sess
         return r;
     };
     size_t cached = 0;
+    // The copies go out in growing batches while the host is still inserting the later
+    // blocks into the index, as in skv_hot_match_restore.
+    size_t batch_pages = 16;
     for (size_t b = 0; b < n_blocks; ++b) {
         const size_t tokens = first_tokens + b * bt;
+        if (pages.size() >= batch_pages) {
+            rc = flush();
+            if (rc) return rc;
+            batch_pages = std::min<size_t>(batch_pages * 5 / 2, COPY_MAX_PAGES);
+        }
         bool skipped = false;
         while (h->free_slots.size() < h->pages_per_block) {
             uint64_t id = 0;
