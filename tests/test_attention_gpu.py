@@ -193,6 +193,46 @@ def test_normal_inputs_config0(state):
     assert delta.max() <= 1e-4, delta.max()
 
 
+@pytest.mark.parametrize("q_scale,k_scale,v_scale,tol", [
+    # Scores in the hundreds and thousands: softmax is nearly one-hot and near-tied keys
+    # trade weight on the last bits of their scores. Against an fp64 evaluation of the same
+    # rows the CPU path and the device are equally far off at |score| ~ 100 (2e-4 each); at
+    # |score| ~ 1000 the device's two-term bf16 query split (2^-17 relative) shows: 1e-3
+    # against the CPU path's 1e-4. The bounds follow that and stay under the contract's 1e-2.
+    (30.0, 30.0, 1.0, 8e-3),
+    (10.0, 10.0, 1.0, 2e-3),
+    (1e-3, 1e-3, 1e4, 8e-4),     # scores ~ 0: uniform weights over large values
+    (8.0, 8.0, 1e-6, 8e-4),      # peaked weights over tiny values (no flush to zero in the product)
+])
+def test_attention_extreme_magnitudes(state, q_scale, k_scale, v_scale, tol):
+    """The online softmax (running maximum, base-2 exponent) and the hi/lo operand split must
+    neither overflow nor lose the answer when scores are huge, vanish, or values are tiny:
+    decode (split context) and a prefill chunk against the CPU path, error relative to the
+    scale of the values."""
+    q_heads, kv_heads, head_dim, n, chunk = 16, 2, 256, 3000, 80
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(5)
+    keys = (rng.standard_normal((n, kv_dim)) * k_scale).astype(np.float32)
+    values = (rng.standard_normal((n, kv_dim)) * v_scale).astype(np.float32)
+    lay = oracle.layout(q_heads, kv_heads, head_dim)
+    cache = oracle.LayerKvCache("bf16r")
+    cache.append_batch(keys, values, lay)
+    kv = state.full_attention_bf16(n + chunk, q_heads, kv_heads, head_dim)
+    kv.seed(keys, values, n)
+    q = (rng.standard_normal(q_dim) * q_scale).astype(np.float32)
+    got = kv.attention_decode(q)
+    want = oracle.cached_attention_one(q, cache, lay)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= tol * v_scale, np.abs(got - want).max()
+    qs = (rng.standard_normal((chunk, q_dim)) * q_scale).astype(np.float32)
+    ks = (rng.standard_normal((chunk, kv_dim)) * k_scale).astype(np.float32)
+    vs = (rng.standard_normal((chunk, kv_dim)) * v_scale).astype(np.float32)
+    got = kv.prefill_rows(qs, ks, vs)
+    want = oracle.cached_attention_prefill_rows(qs, ks, vs, cache, lay)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= tol * v_scale, np.abs(got - want).max()
+
+
 # ---- chunked prefill over the cache (multi-query, matrix cores) ----------------------------
 @pytest.fixture(params=["by-shape", "one-tile", "two-tiles"])
 def tiles_per_wavefront(request):
