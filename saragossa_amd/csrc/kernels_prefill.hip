@@ -395,19 +395,31 @@ __global__ __launch_bounds__(256) void merge_rows_kernel(DecodeArgs a) {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float lsum = 0.0f;
     const bool vec_ok = (g.head_dim & 3) == 0;
-    for (int sp = 0; sp < a.splits_total; ++sp) {
-        const long pidx = base + (long)sp * n_slots;
-        const float w = fast_exp2(a.part_m[pidx] - m_safe);
-        lsum += w * a.part_l[pidx];
-        const float *po = a.part_o + pidx * g.head_dim + c4;
-        if (vec_ok) {
-            const float4_t v = *reinterpret_cast<const float4_t *>(po);
+    // four splits per round: their loads are all issued before the first is consumed (the
+    // partials are read once: non-temporal)
+    for (int sp0 = 0; sp0 < a.splits_total; sp0 += 4) {
+        float w[4], lp[4];
+        float4_t v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] += w * v[i];
-        } else {
+        for (int u = 0; u < 4; ++u) {
+            const int sp = min(sp0 + u, a.splits_total - 1); // a repeat of the last one weighs zero below
+            const long pidx = base + (long)sp * n_slots;
+            w[u] = a.part_m[pidx];
+            lp[u] = a.part_l[pidx];
+            const float *po = a.part_o + pidx * g.head_dim + c4;
+            if (vec_ok) {
+                v[u] = __builtin_nontemporal_load(reinterpret_cast<const float4_t *>(po));
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (c4 + i < g.head_dim) acc[i] += w * po[i];
+                for (int i = 0; i < 4; ++i) v[u][i] = c4 + i < g.head_dim ? po[i] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float wu = sp0 + u < a.splits_total ? fast_exp2(w[u] - m_safe) : 0.0f;
+            lsum += wu * lp[u];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += wu * v[u][i];
         }
     }
     float *dst = a.out + ((long)(slot / g.gqa) * g.q_heads + kvh * g.gqa + slot % g.gqa) * g.head_dim + c4;
