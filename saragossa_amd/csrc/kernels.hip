@@ -18,21 +18,67 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
 
 // ------------------------------------------------------------------------------------
 // append: f32 rows -> bf16 tiles. One thread per (row, kv head, 8-dim group): a 16-byte
-// store into the K tile, eight 2-byte stores into the transposed V tile.
+// store into the K tile, eight 2-byte stores into the transposed V tile. In a batch, the
+// rows that form whole position-aligned groups of four take a second kind of work item for
+// V instead: one thread per (row group, kv head, 32-dim block, column) gathers 4 rows x 2
+// dims and writes the 16 contiguous bytes they occupy in the tile.
 // Stands in for copy_at_f32_to_bf16 (src/decode_resident/kernels.rs:1036-1044).
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void append_kernel(AppendArgs a) {
     const Geom g = a.g;
     const int groups = (g.head_dim + 7) >> 3;
     const long per_row = (long)g.kv_heads * groups;
-    const long total = per_row * a.n_rows;
+    const long page0 = a.first_pos >> 4; // first page of positions the batch touches
+    const long n_blk = ((a.first_pos + a.n_rows + 15) >> 4) - page0;
+    const long total_rows = a.by_page ? n_blk * per_row * 16 : per_row * a.n_rows;
     const int kv_dim = g.kv_heads * g.head_dim;
+    const int per_grp = g.kv_heads * (g.P >> 5) * 16;
+    const long total = total_rows + (long)(a.v_grp_rows >> 2) * per_grp;
     for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total;
          t += (long)gridDim.x * blockDim.x) {
-        const int row = (int)(t / per_row);
-        const int rem = (int)(t - (long)row * per_row);
-        const int kvh = rem / groups;
-        const int grp = rem - kvh * groups;
+        if (t >= total_rows) {
+            // V of one aligned group of four rows: columns c and c + 16 of a 32-dim block
+            const long u = t - total_rows;
+            const int grp4 = (int)(u / per_grp);
+            int rem = (int)(u - (long)grp4 * per_grp);
+            const int kvh = rem / ((g.P >> 5) * 16);
+            rem -= kvh * ((g.P >> 5) * 16);
+            const int db = rem >> 4, c = rem & 15;
+            const int row0 = a.v_grp_first + grp4 * 4;
+            const long slot = slot_of(a.first_pos + row0, g.ring_rows); // a multiple of 4
+            const int page = a.table[slot >> 4];
+            const long tile = (long)page * g.page_elems + (long)kvh * g.tile_elems;
+            const int d0 = db * 32 + c, d1 = d0 + 16;
+            const float *vs = a.v_src + (long)row0 * kv_dim + kvh * g.head_dim;
+            uint16_t lo[4], hi[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                lo[r] = d0 < g.head_dim ? bf16_bits(vs[(long)r * kv_dim + d0]) : (uint16_t)0;
+                hi[r] = d1 < g.head_dim ? bf16_bits(vs[(long)r * kv_dim + d1]) : (uint16_t)0;
+            }
+            uint4 pk;
+            pk.x = lo[0] | ((uint32_t)lo[1] << 16);
+            pk.y = lo[2] | ((uint32_t)lo[3] << 16);
+            pk.z = hi[0] | ((uint32_t)hi[1] << 16);
+            pk.w = hi[2] | ((uint32_t)hi[3] << 16);
+            *reinterpret_cast<uint4 *>(a.v_pool + tile + v_index(g.P, (int)(slot & 15), d0)) = pk;
+            continue;
+        }
+        int row, kvh, grp;
+        if (a.by_page) {
+            const long blk = t / (per_row * 16);
+            const int rem = (int)(t - blk * per_row * 16);
+            const long pos = (page0 + blk) * 16 + (rem & 15);
+            if (pos < a.first_pos || pos >= a.first_pos + a.n_rows) continue;
+            row = (int)(pos - a.first_pos);
+            grp = (rem >> 4) % groups;
+            kvh = (rem >> 4) / groups;
+        } else {
+            row = (int)(t / per_row);
+            const int rem = (int)(t - (long)row * per_row);
+            kvh = rem / groups;
+            grp = rem - kvh * groups;
+        }
         const long slot = slot_of(a.first_pos + row, g.ring_rows);
         const int page = a.table[slot >> 4];
         const int r = (int)(slot & 15);
@@ -50,6 +96,7 @@ __global__ __launch_bounds__(256) void append_kernel(AppendArgs a) {
         pk.z = kb[4] | ((uint32_t)kb[5] << 16);
         pk.w = kb[6] | ((uint32_t)kb[7] << 16);
         *reinterpret_cast<uint4 *>(a.k_pool + tile + k_index(g.P, r, d0)) = pk;
+        if (row >= a.v_grp_first && row < a.v_grp_first + a.v_grp_rows) continue; // V by groups
 #pragma unroll
         for (int e = 0; e < 8; ++e)
             if (e < nd) a.v_pool[tile + v_index(g.P, r, d0 + e)] = bf16_bits(vs[e]);
@@ -58,7 +105,10 @@ __global__ __launch_bounds__(256) void append_kernel(AppendArgs a) {
 
 hipError_t launch_append(const AppendArgs &a, hipStream_t s) {
     const int groups = (a.g.head_dim + 7) >> 3;
-    const long total = (long)a.g.kv_heads * groups * a.n_rows;
+    const long n_blk = ((a.first_pos + a.n_rows + 15) >> 4) - (a.first_pos >> 4);
+    const long row_items = a.by_page ? n_blk * 16 : (long)a.n_rows;
+    const long total = (long)a.g.kv_heads * groups * row_items +
+                       (long)(a.v_grp_rows >> 2) * a.g.kv_heads * (a.g.P >> 5) * 16;
     if (total <= 0) return hipSuccess;
     long blocks = (total + 255) / 256;
     if (blocks > 65535 * 4) blocks = 65535 * 4;

@@ -323,6 +323,13 @@ int32_t encode_append(skv_layer *L, hipStream_t s, const float *k_dev, const flo
         a.first_pos += (long)skip;
         a.n_rows = L->g.ring_rows;
     }
+    // whole groups of four rows at positions that are multiples of 4 write V in 16-byte units
+    if (a.n_rows >= 8) {
+        a.by_page = 1;
+        const long lead = (4 - (a.first_pos & 3)) & 3;
+        a.v_grp_first = (int)lead;
+        a.v_grp_rows = (int)((a.n_rows - lead) & ~3L);
+    }
     SKV_HIP(launch_append(a, s));
     L->len += n_rows;
     if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)

@@ -86,6 +86,14 @@ struct AppendArgs {
     const int32_t *table;
     long first_pos; // position of the first appended row
     int n_rows;
+    // rows [v_grp_first, v_grp_first + v_grp_rows) of the batch start at a position that is a
+    // multiple of 4 and come in whole groups of 4: their V elements are written as 16-byte
+    // units of the transposed tile (4 rows x 2 dims) instead of 2-byte stores
+    int v_grp_first;
+    int v_grp_rows;
+    // batches: row items are numbered page by page with the row inside the page fastest, so
+    // that sixteen neighbouring threads write 256 contiguous bytes of a K tile
+    int by_page;
     Geom g;
 };
 
