@@ -264,10 +264,125 @@ __global__ __launch_bounds__(256) void norm_rope_kernel(NormRopeArgs a) {
                            a.rope_style);
 }
 
+// The same for many rows (a prefill chunk): one workgroup per ROWS_PAIRS (row, head) pairs.
+// Their raw values are staged in LDS with coalesced loads (pair stride head_dim + 1: lane i
+// walking pair i is conflict-free), lane i of the first wavefront takes the sum of squares of
+// pair i in index order, exactly as above, and all threads then produce the outputs with
+// coalesced stores, weight and rotations read from LDS. One workgroup per pair, as for a
+// single row, leaves 255 of 256 lanes waiting for the ordered sum: 24.6 us for 512 rows of
+// 32 heads x 128 against 14.5 us this way, 89.8 against 32.8 us for 2048 rows. Sixteen pairs
+// per workgroup are best up to head_dim 128, eight above (measured).
+template <int ROWS_PAIRS>
+__global__ __launch_bounds__(256) void norm_rope_rows_kernel(NormRopeArgs a) {
+    // [pairs][head_dim + 1] values | [pairs] inverse rms | [head_dim] weight | [rows][rope_dims] rotations
+    extern __shared__ float rows_lds[];
+    const int hd = a.head_dim;
+    const int stride = hd + 1;
+    float *inv_s = rows_lds + ROWS_PAIRS * stride;
+    float *w_s = inv_s + ROWS_PAIRS;
+    float *rope_s = w_s + hd;
+    const int lane = threadIdx.x; // 0..255; the ordered sums use the first ROWS_PAIRS
+    const long n_pairs = (long)a.n_rows * a.heads;
+    const long pair0 = (long)blockIdx.x * ROWS_PAIRS;
+    const int here = (int)min((long)ROWS_PAIRS, n_pairs - pair0);
+    const long row_elems = (long)a.heads * hd;
+    const int hstride = a.x_head_stride > 0 ? a.x_head_stride : hd;
+    // threads per pair: a power of two that covers head_dim in at most two passes, so that a
+    // thread's (pair, column) comes from shifts and masks, not divisions
+    const int tpp_log = hd > 128 ? 8 : hd > 64 ? 7 : 6;
+    const int tpp = 1 << tpp_log, ppi = 256 >> tpp_log;
+    const int sub = lane >> tpp_log, c0 = lane & (tpp - 1);
+    // eight pairs' loads are issued before the first is stored (unconditional, from clamped
+    // indices): the staging is then a few memory round trips instead of one per pair
+    constexpr int U = 8;
+    for (int pb = sub; pb < here; pb += ppi * U) {
+        float v0[U], v1[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int pair = (int)pair0 + min(pb + u * ppi, here - 1);
+            const int r = pair / a.heads;
+            const int h = pair - r * a.heads;
+            const float *src = a.x + (long)r * row_elems + (long)h * hstride;
+            v0[u] = src[min(c0, hd - 1)];
+            v1[u] = src[min(c0 + tpp, hd - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int p = pb + u * ppi;
+            if (p < here) {
+                if (c0 < hd) rows_lds[p * stride + c0] = v0[u];
+                if (c0 + tpp < hd) rows_lds[p * stride + c0 + tpp] = v1[u];
+            }
+        }
+    }
+    // the weight and the rotations of the rows this workgroup touches: read per element below,
+    // from LDS instead of one dependent global load each
+    const long r_first = pair0 / a.heads;
+    const int n_r = (int)((pair0 + here - 1) / a.heads - r_first) + 1;
+    if (a.weight)
+        for (int c = lane; c < hd; c += 256) w_s[c] = a.weight[c];
+    if (a.rope)
+        for (int e = lane; e < n_r * a.rope_dims; e += 256) rope_s[e] = a.rope[r_first * a.rope_dims + e];
+    __syncthreads();
+    if (lane < here) {
+        // head_inv_rms over the lane's own pair, sixteen LDS reads in flight per round; the
+        // multiplications and additions are the same, in the same order
+        const float *row = rows_lds + lane * stride;
+        float inv = 1.0f;
+        if (a.weight) {
+#pragma clang fp contract(off)
+            float sum = 0.0f;
+            int c = 0;
+            for (; c + 16 <= hd; c += 16) {
+                float v[16];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) v[j] = row[c + j];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const float sq = v[j] * v[j];
+                    sum = sum + sq;
+                }
+            }
+            for (; c < hd; ++c) {
+                const float sq = row[c] * row[c];
+                sum = sum + sq;
+            }
+            const float mean_square = sum / (float)hd;
+            inv = 1.0f / sqrtf(mean_square + a.eps);
+        }
+        inv_s[lane] = inv;
+    }
+    __syncthreads();
+    for (int p = sub; p < here; p += ppi) {
+        const int pair = (int)pair0 + p;
+        const int r = pair / a.heads;
+        const float *rope_row = a.rope ? rope_s + (r - r_first) * a.rope_dims : nullptr;
+        const float inv = inv_s[p];
+        for (int c = c0; c < hd; c += tpp)
+            a.out[(long)pair * hd + c] = norm_rope_elem(rows_lds + p * stride, c, inv, a.weight ? w_s : nullptr,
+                                                  rope_row, a.rope_dims, a.rope_style);
+    }
+}
+
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s) {
     if (a.heads <= 0 || a.head_dim <= 0 || a.head_dim > 512) return hipErrorInvalidValue;
     const int rows = a.n_rows > 0 ? a.n_rows : 1;
     if (rows > 65535) return hipErrorInvalidValue;
+    if (rows >= 4) {
+        const int pairs = a.head_dim <= 128 ? 16 : 8;
+        const int rows_per_wg = std::min(rows, (pairs + a.heads - 1) / a.heads + 1);
+        const size_t lds = (size_t)(pairs * (a.head_dim + 1) + pairs + a.head_dim +
+                                    (a.rope ? (size_t)rows_per_wg * a.rope_dims : 0)) * sizeof(float);
+        const long n_pairs = (long)rows * a.heads;
+        NormRopeArgs b = a;
+        b.n_rows = rows;
+        const dim3 grid((unsigned)((n_pairs + pairs - 1) / pairs));
+        if (pairs == 16)
+            hipLaunchKernelGGL(norm_rope_rows_kernel<16>, grid, dim3(256), lds, s, b);
+        else
+            hipLaunchKernelGGL(norm_rope_rows_kernel<8>, grid, dim3(256), lds, s, b);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(norm_rope_kernel, dim3((unsigned)a.heads, (unsigned)rows), dim3(256), 0, s, a);
     return hipGetLastError();
 }

@@ -64,23 +64,28 @@ def test_rms_norm_rope_decode_is_bit_exact_on_random_rows(state, heads, head_dim
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("heads,head_dim,rope_dims,theta,offset,rows", [
-    (32, 128, 128, 1.0e6, 1536, 512),   # a prefill chunk of config 1's q rows
-    (2, 256, 64, 1.0e7, 32760, 20),     # partial rotary across a page boundary
-    (3, 40, 20, 10000.0, 0, 7),
+@pytest.mark.parametrize("heads,head_dim,rope_dims,theta,offset,rows,style", [
+    (32, 128, 128, 1.0e6, 1536, 512, 0),   # a prefill chunk of config 1's q rows
+    (2, 256, 64, 1.0e7, 32760, 20, 0),     # partial rotary across a page boundary
+    (3, 40, 20, 10000.0, 0, 7, 0),
+    (16, 256, 256, 1.0e6, 0, 130, 0),      # config 2's q rows: eight (row, head) pairs per workgroup
+    (1, 512, 512, 10000.0, 5, 9, 0),       # one head: every pair of a workgroup is another row
+    (5, 64, 32, 10000.0, 100, 33, 1),      # interleaved pairs, four pairs per pass of the workgroup
+    (8, 128, 128, 1.0e6, 11, 3, 0),        # under four rows: one workgroup per (row, head)
 ])
-def test_rms_norm_rope_rows_is_bit_exact(state, heads, head_dim, rope_dims, theta, offset, rows):
+def test_rms_norm_rope_rows_is_bit_exact(state, heads, head_dim, rope_dims, theta, offset, rows, style):
     """A chunk of rows at consecutive positions == rms_norm_rope_heads_at on a [seq, dim] tensor
     with position_offset (src/decoder/attention_ops.rs:682-777)."""
     rng = np.random.default_rng(rows)
     x = rng.standard_normal((rows, heads * head_dim), dtype=np.float32) * 2
     w = (0.5 + rng.random(head_dim, dtype=np.float32)).astype(np.float32)
-    rope = state.rope_table(offset + rows, rope_dims, theta)
+    rope = state.rope_table(offset + rows, rope_dims, theta, style=style)
     xd, wd = _dev(x), _dev(w)
     out = torch.empty_like(xd)
     state.encode_rms_norm_rope_rows(_stream(), rope, offset, xd.data_ptr(), wd.data_ptr(), rows, heads,
                                     head_dim, 1e-6, out.data_ptr())
-    want = oracle.rms_norm_rope_heads_at(x, heads, head_dim, rope_dims, w, 1e-6, theta, offset)
+    want = oracle.rms_norm_rope_heads_at(x, heads, head_dim, rope_dims, w, 1e-6, theta, offset,
+                                         style=oracle.ROPE_INTERLEAVED if style else oracle.ROPE_HALVES)
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
     with pytest.raises(skv.DimensionError):   # the last row's position is outside the table
         state.encode_rms_norm_rope_rows(_stream(), rope, offset + 1, xd.data_ptr(), wd.data_ptr(), rows,
