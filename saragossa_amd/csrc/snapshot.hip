@@ -248,13 +248,23 @@ struct skv_hot {
     // counters (x-saragossa-reused-prefix-tokens accounting and eviction log, serve/state.rs:59-80, 263-266)
     uint64_t evictions = 0;
     uint64_t skipped = 0;
+    // State buffers of evicted entries, kept for the next remember of the same shapes: an
+    // eviction then costs neither a device synchronisation nor a free, a remember no
+    // allocation (copies into and out of them are ordered by the stream, like the page slots).
+    std::vector<skv_snapshot *> spare_states;
 };
+constexpr size_t HOT_MAX_SPARE_STATES = 4;
 
 static void hot_release(skv_hot *h, uint64_t id) {
     auto it = h->entries.find(id);
     if (it == h->entries.end()) return;
     for (int32_t s : it->second.slots) h->free_slots.push_back(s);
-    if (it->second.state) skv_snapshot_free(it->second.state);
+    if (it->second.state) {
+        if (h->spare_states.size() < HOT_MAX_SPARE_STATES)
+            h->spare_states.push_back(it->second.state);
+        else
+            skv_snapshot_free(it->second.state);
+    }
     h->entries.erase(it);
 }
 
@@ -478,6 +488,7 @@ void skv_hot_destroy(skv_hot *h) {
     (void)hipDeviceSynchronize();
     for (auto &kv : h->entries)
         if (kv.second.state) skv_snapshot_free(kv.second.state);
+    for (skv_snapshot *sp : h->spare_states) skv_snapshot_free(sp);
     if (h->pool) (void)hipFree(h->pool);
     delete h->index;
     delete h;
@@ -559,8 +570,32 @@ int32_t skv_hot_remember(skv_hot *h, skv_stream stream, const uint8_t session[32
     }
     rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), e.slots.data(),
                     h->pages_per_block, nullptr, true, as_stream(stream));
-    if (!rc && n_states)
-        rc = skv_state_snapshot(h->ctx, stream, state_ptrs, state_bytes, n_states, &e.state);
+    if (!rc && n_states) {
+        // a spare buffer of the same shapes, if an eviction left one
+        for (size_t i = 0; i < h->spare_states.size() && !e.state; ++i) {
+            skv_snapshot *sp = h->spare_states[i];
+            if (sp->sizes.size() == n_states && state_bytes && std::equal(sp->sizes.begin(), sp->sizes.end(), state_bytes)) {
+                e.state = sp;
+                h->spare_states.erase(h->spare_states.begin() + (long)i);
+            }
+        }
+        if (e.state) {
+            bool ok = state_ptrs != nullptr;
+            std::vector<void *> dst(n_states);
+            for (size_t i = 0; i < n_states && ok; ++i) {
+                ok = state_ptrs[i] != nullptr;
+                dst[i] = e.state->base + e.state->offsets[i];
+            }
+            rc = ok ? launch_flat(state_ptrs, dst.data(), state_bytes, n_states, as_stream(stream))
+                    : fail(SKV_ERR_DEVICE, "state_snapshot: pointeur nul");
+            if (rc) {
+                h->spare_states.push_back(e.state);
+                e.state = nullptr;
+            }
+        } else {
+            rc = skv_state_snapshot(h->ctx, stream, state_ptrs, state_bytes, n_states, &e.state);
+        }
+    }
     if (rc) {
         for (int32_t s : e.slots) h->free_slots.push_back(s);
         return rc;

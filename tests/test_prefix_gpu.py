@@ -248,6 +248,23 @@ def test_hot_cache_with_recurrent_state_and_skip_when_nothing_to_evict(state):
     assert reused == 32 and h == h2
     assert torch.equal(out, torch.arange(4096, dtype=torch.float32, device="cuda") + 1.0)
     check_contents(fresh, 32, tokens, kv_dim)
+    # a pool of one block: remembering another session's block evicts the first and takes over
+    # its state buffer; what is restored afterwards is the newcomer's state, byte for byte
+    solo = skv.HotCache(state, bt, 8, 1, layers)
+    assert solo.remember_prefix_block(root, h1, 16, layers, [ssm.data_ptr()], [ssm.numel() * 4])
+    other_root = BlockHash.for_session("another session")
+    g1 = BlockHash.chain(other_root, tokens[:16])
+    ssm += 5.0
+    assert solo.remember_prefix_block(other_root, g1, 16, layers, [ssm.data_ptr()], [ssm.numel() * 4])
+    assert solo.evictions() == 1 and len(solo) == 1
+    again = make_layers(state, 2, 64, dims, seed=11)
+    out.zero_()
+    reused, _ = solo.match_restore(other_root, tokens, again, [out.data_ptr()], [out.numel() * 4])
+    torch.cuda.synchronize()
+    assert reused == 16 and torch.equal(out, ssm)
+    check_contents(again, 16, tokens, kv_dim)
+    reused, _ = solo.match_restore(root, tokens, again, [out.data_ptr()], [out.numel() * 4])
+    assert reused == 0                                        # the evicted block is gone
     # a disabled cache (capacity 0) and a pool with no room and nothing to evict both skip silently
     off = skv.HotCache(state, bt, 0, 2, layers)
     assert not off.remember_prefix_block(root, h1, 16, layers)
