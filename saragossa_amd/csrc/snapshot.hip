@@ -85,41 +85,70 @@ __global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
 
 // ---- flat copies of several device buffers in one launch (recurrent state) ----------------
 constexpr int FLAT_MAX = 120;
+constexpr uint32_t FLAT_CHUNK16 = 2048; // 16-byte words per workgroup: 32 KiB, eight per thread
 struct FlatArgs {
     const uint8_t *src[FLAT_MAX];
     uint8_t *dst[FLAT_MAX];
     uint64_t bytes[FLAT_MAX];
+    uint32_t first_chunk[FLAT_MAX + 1]; // running count of 32 KiB chunks: buffer i owns [first_chunk[i], first_chunk[i+1])
     int n;
 };
 
-// grid (chunks, buffers): the workgroups of a buffer stride over it together
+// One workgroup per 32 KiB chunk of one buffer (a buffer of 96 KiB gets three workgroups, one
+// of 2 MiB sixty-four: none idles and none loops), eight non-temporal 16-byte loads in flight
+// per thread, then the stores.
 __global__ __launch_bounds__(256) void flat_copy_kernel(FlatArgs a) {
-    const int b = blockIdx.y;
+    const uint32_t chunk = blockIdx.x;
+    int lo = 0, hi = a.n - 1; // the buffer that owns the chunk (uniform: scalar loads)
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (a.first_chunk[mid] <= chunk) lo = mid; else hi = mid - 1;
+    }
+    const int b = lo;
     const uint64_t n = a.bytes[b];
     const long n16 = (long)(n >> 4);
-    copy_stream(reinterpret_cast<const u32x4 *>(a.src[b]), reinterpret_cast<u32x4 *>(a.dst[b]), n16,
-                (long)blockIdx.x * 256 + threadIdx.x, (long)gridDim.x * 256);
-    if (blockIdx.x == 0) // tail bytes of a buffer whose size is not a multiple of 16
+    const long w0 = (long)(chunk - a.first_chunk[b]) * FLAT_CHUNK16;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(a.src[b]);
+    u32x4 *dst = reinterpret_cast<u32x4 *>(a.dst[b]);
+    const long end = min(w0 + (long)FLAT_CHUNK16, n16);
+    if (w0 + (long)FLAT_CHUNK16 <= n16) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + w0 + u * 256 + threadIdx.x);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], dst + w0 + u * 256 + threadIdx.x);
+    } else {
+        for (long i = w0 + threadIdx.x; i < end; i += 256) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+    }
+    if (end == n16) // the chunk that ends the buffer also copies its last bytes, if any
         for (uint64_t i = ((uint64_t)n16 << 4) + threadIdx.x; i < n; i += 256) a.dst[b][i] = a.src[b][i];
 }
 
 static int32_t launch_flat(const void *const *src, void *const *dst, const size_t *bytes, size_t n,
                            hipStream_t s) {
-    for (size_t first = 0; first < n; first += FLAT_MAX) {
+    size_t first = 0;
+    while (first < n) {
         FlatArgs a{};
-        a.n = (int)std::min<size_t>(FLAT_MAX, n - first);
-        uint64_t largest = 0;
-        for (int i = 0; i < a.n; ++i) {
-            a.src[i] = (const uint8_t *)src[first + i];
-            a.dst[i] = (uint8_t *)dst[first + i];
-            a.bytes[i] = bytes[first + i];
-            if (((uintptr_t)a.src[i] | (uintptr_t)a.dst[i]) & 15)
+        uint64_t chunks = 0;
+        int k = 0;
+        // as many buffers as fit the argument block and a 32-bit chunk count
+        for (; k < FLAT_MAX && first + k < n; ++k) {
+            const uint64_t c = std::max<uint64_t>((((uint64_t)bytes[first + k] >> 4) + FLAT_CHUNK16 - 1) / FLAT_CHUNK16, 1);
+            if (chunks + c > 0x7fffffffull) break;
+            a.src[k] = (const uint8_t *)src[first + k];
+            a.dst[k] = (uint8_t *)dst[first + k];
+            a.bytes[k] = bytes[first + k];
+            if (((uintptr_t)a.src[k] | (uintptr_t)a.dst[k]) & 15)
                 return fail(SKV_ERR_DEVICE, "copie d'état: pointeur non aligné sur 16 octets");
-            largest = std::max<uint64_t>(largest, a.bytes[i]);
+            a.first_chunk[k] = (uint32_t)chunks;
+            chunks += c;
         }
-        const unsigned chunks = (unsigned)std::min<uint64_t>(std::max<uint64_t>((largest + 32767) / 32768, 1), 1024);
-        hipLaunchKernelGGL(flat_copy_kernel, dim3(chunks, (unsigned)a.n), dim3(256), 0, s, a);
+        if (k == 0) return fail(SKV_ERR_DIMENSION, "copie d'état: tampon trop grand pour un lancement");
+        a.first_chunk[k] = (uint32_t)chunks;
+        a.n = k;
+        hipLaunchKernelGGL(flat_copy_kernel, dim3((unsigned)chunks), dim3(256), 0, s, a);
         SKV_HIP(hipGetLastError());
+        first += (size_t)k;
     }
     return SKV_OK;
 }
