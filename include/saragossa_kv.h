@@ -43,7 +43,14 @@ typedef struct skv_snapshot skv_snapshot;
 typedef struct skv_prefix skv_prefix;
 typedef struct skv_hot skv_hot;
 
-/* A stream argument is a hipStream_t passed as void*; NULL is the default stream. */
+/* A stream argument is a hipStream_t passed as void*; NULL is the default stream.
+ * The *_device entry points only queue work on that stream: they neither wait for the
+ * device nor switch devices, so the stream must belong to the context's device and that
+ * device must be current on the calling thread (the *_host entry points and the create /
+ * destroy calls make it current themselves). Host-side bookkeeping (len, ring position)
+ * advances when the call returns, before the device has run the work, exactly like the
+ * reference's encode-time `len += 1` (src/decode_resident/attention.rs:993); buffers handed
+ * to a *_device call must stay valid until the stream has passed that work. */
 typedef void *skv_stream;
 
 /* ---- errors, version ---------------------------------------------------- */
