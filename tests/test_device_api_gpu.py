@@ -272,3 +272,42 @@ def test_prefill_chunk_device_with_unaligned_query_pointer(state):
         assert np.abs(got - want).max() <= 1e-4
         results.append(got)
     assert np.array_equal(results[0], results[1]) and np.array_equal(results[0], results[2])
+
+
+def test_attention_launches_replay_correctly_from_a_hip_graph(state):
+    """The *_device entry points only queue kernels (no allocation, no synchronisation, no
+    memset), so a caller may capture them in a HIP graph; what is captured is the work at the
+    lengths of capture time. Several layers' attention captured once, replayed three times
+    with eager work and synchronisations in between, each replay against the eager result
+    (short context: single split; long context: split + merge)."""
+    q_heads, kv_heads, head_dim = 16, 2, 256
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(21)
+    layers = []
+    for n in (100, 5000, 900):
+        kv = state.full_attention_bf16(n, q_heads, kv_heads, head_dim)
+        kv.seed(rng.standard_normal((n, kv_dim), dtype=np.float32),
+                rng.standard_normal((n, kv_dim), dtype=np.float32), n)
+        layers.append(kv)
+    q = _dev(rng.standard_normal(q_dim, dtype=np.float32))
+    outs = [torch.zeros(q_dim, device="cuda") for _ in layers]
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):      # warm up outside the capture (lazy kernel attributes)
+        for kv, o in zip(layers, outs):
+            kv.encode_attention_decode(side.cuda_stream, q.data_ptr(), o.data_ptr())
+    torch.cuda.synchronize()
+    eager = [o.clone() for o in outs]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for kv, o in zip(layers, outs):
+            kv.encode_attention_decode(side.cuda_stream, q.data_ptr(), o.data_ptr())
+    for replay in range(3):
+        for o in outs:
+            o.fill_(float(replay))                                      # eager work between replays
+        layers[0].encode_attention_decode(_stream(), q.data_ptr(), outs[0].data_ptr())
+        torch.cuda.synchronize()
+        outs[0].zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, e in zip(outs, eager):
+            assert torch.equal(o, e), f"replay {replay}"
