@@ -57,6 +57,16 @@ def test_config2_hybrid_32k_decode_steps(state):
             want = oracle.decode_step(caches[li], kn[t, li], vn[t, li], qn[t, li], lay)
             worst = max(worst, float(np.abs(got[t, li] - want).max()))
     assert worst <= 1e-4, worst
+    # an implementation that shares nothing with the oracle: the last step of layer 0 again
+    # as textbook softmax attention in float64 (torch, on the device) over the rows read back
+    # from the cache
+    gk, gv = layers[0].read_rows_f32()
+    K = torch.from_numpy(gk).cuda().double().view(ctx + steps, kvh, hd)
+    V = torch.from_numpy(gv).cuda().double().view(ctx + steps, kvh, hd)
+    qd = qs[steps - 1, 0].double().view(kvh, qh // kvh, hd)
+    p = torch.softmax(torch.einsum("kgd,nkd->kgn", qd, K) / hd ** 0.5, dim=-1)
+    ref = torch.einsum("kgn,nkd->kgd", p, V).reshape(-1)
+    assert float((out[steps - 1, 0].double() - ref).abs().max()) <= 1e-5
     for kv, c in zip(layers, caches):
         gk, gv = kv.read_rows_f32(ctx - 40, 40 + steps)
         assert np.array_equal(gk, c.keys()[ctx - 40:]) and np.array_equal(gv, c.values()[ctx - 40:])
