@@ -136,6 +136,21 @@ def test_config4_sliding_window_model_batch1_and_batch4(state):
     assert layers[0].pages() == window // 16 and layers[5].pages() == (ctx + 4 + 15) // 16
     gk, _ = layers[0].read_rows_f32(layers[0].len() - window, window)
     assert np.array_equal(gk, caches[0].keys()[-window:])
+    # independent of the oracle: one more attention over the global layer (all 65540 rows) and
+    # over a ring layer (its last 1024 rows) against float64 softmax attention in torch
+    for li in (5, 0):
+        kv = layers[li]
+        n = kv.len()
+        first = 0 if li == 5 else n - window
+        gk, gv = kv.read_rows_f32(first, n - first)
+        K = torch.from_numpy(gk).cuda().double().view(n - first, kvh, hd)
+        V = torch.from_numpy(gv).cuda().double().view(n - first, kvh, hd)
+        q = torch.randn(q_dim, device="cuda", generator=gen)
+        o = torch.empty(q_dim, device="cuda")
+        kv.encode_attention_decode_windowed(_stream(), q.data_ptr(), o.data_ptr(), first)
+        p = torch.softmax(torch.einsum("kgd,nkd->kgn", q.double().view(kvh, qh // kvh, hd), K) / hd ** 0.5, dim=-1)
+        ref = torch.einsum("kgn,nkd->kgd", p, V).reshape(-1)
+        assert float((o.double() - ref).abs().max()) <= 1e-5, li
     for kv in layers:
         kv.close()
     four = [build_sequence(3) for _ in range(4)]
