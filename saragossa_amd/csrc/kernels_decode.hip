@@ -140,11 +140,21 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     const int pb_new = a.new_slot >> 4;
     const int r_new = a.new_slot & 15;
     const bool appends = a.k_new != nullptr && C == 1 && pb_new >= pb0 && pb_new < pb1;
-    float k_row = 0.0f, v_row = 0.0f; // element tid of the new row of this kv head
-    if (appends && tid < g.head_dim) {
-        k_row = a.k_new[kvh * g.head_dim + tid];
-        v_row = a.v_new[kvh * g.head_dim + tid];
+    // elements tid (and tid + THREADS where the head is wider than the workgroup) of the new
+    // row of this kv head
+    constexpr int NE = (P + THREADS - 1) / THREADS;
+    static_assert(!PRE || NE == 1, "the fused pre-KV step keeps one row element per thread");
+    float k_rows[NE], v_rows[NE];
+#pragma unroll
+    for (int u = 0; u < NE; ++u) {
+        k_rows[u] = 0.0f;
+        v_rows[u] = 0.0f;
+        if (appends && tid + u * THREADS < g.head_dim) {
+            k_rows[u] = a.k_new[kvh * g.head_dim + tid + u * THREADS];
+            v_rows[u] = a.v_new[kvh * g.head_dim + tid + u * THREADS];
+        }
     }
+    float &k_row = k_rows[0];
     // PRE: raw query rows of the group (and the raw k row, already in k_row)
     constexpr int PRE_U = PRE ? (16 * P + THREADS - 1) / THREADS : 1;
     float pre_q[PRE_U];
@@ -253,16 +263,20 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     if (appends) {
         const int page = a.table[pb_new];
         const long tile_at = (long)page * g.page_elems + (long)kvh * g.tile_elems;
-        if (tid < P) {
-            uint16_t kb = 0, vb = 0;
-            if (tid < g.head_dim) {
-                kb = bf16_bits(k_row);
-                vb = bf16_bits(v_row);
-                const_cast<uint16_t *>(a.k_pool)[tile_at + k_index(P, r_new, tid)] = kb;
-                const_cast<uint16_t *>(a.v_pool)[tile_at + v_index(P, r_new, tid)] = vb;
+#pragma unroll
+        for (int u = 0; u < NE; ++u) {
+            const int d = tid + u * THREADS;
+            if (d < P) {
+                uint16_t kb = 0, vb = 0;
+                if (d < g.head_dim) {
+                    kb = bf16_bits(k_rows[u]);
+                    vb = bf16_bits(v_rows[u]);
+                    const_cast<uint16_t *>(a.k_pool)[tile_at + k_index(P, r_new, d)] = kb;
+                    const_cast<uint16_t *>(a.v_pool)[tile_at + v_index(P, r_new, d)] = vb;
+                }
+                new_k[d] = kb;
+                new_v[d] = vb;
             }
-            new_k[tid] = kb;
-            new_v[tid] = vb;
         }
     }
     if (PRE) {
@@ -636,10 +650,20 @@ static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
     return a.pre ? launch_split_mq<P, WAVES, false, true>(a, s) : launch_split_mq<P, WAVES, false, false>(a, s);
 }
 
+// head_dim 257..512 (global layers of Gemma-4-style models, src/config/accessors.rs:118-123):
+// the accumulators and one K and one V page alone are 256 registers, so the workgroup has
+// four wavefronts, one per SIMD with 512 registers each; no fused pre-KV variant.
+static hipError_t launch_split_wide(const DecodeArgs &a, hipStream_t s) {
+    if (a.pre) return hipErrorInvalidValue;
+    if (a.n_queries > 1 || a.g.gqa > 16) return launch_split_mq<512, 4, true, false>(a, s);
+    return launch_split_mq<512, 4, false, false>(a, s);
+}
+
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     hipError_t e = hipErrorInvalidValue;
     const bool w8 = a.waves == 8;
     switch (a.g.P) {
+    case 512: e = launch_split_wide(a, s); break;
     case 32: e = w8 ? launch_split<32, 8>(a, s) : launch_split<32, 4>(a, s); break;
     case 64: e = w8 ? launch_split<64, 8>(a, s) : launch_split<64, 4>(a, s); break;
     case 128: e = w8 ? launch_split<128, 8>(a, s) : launch_split<128, 4>(a, s); break;
@@ -690,6 +714,7 @@ hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t 
     hipError_t e = hipErrorInvalidValue;
     const bool w8 = a0.waves == 8;
     switch (a0.g.P) {
+    case 512: e = launch_split_batch<512, 4>(b, n_seq, max_splits, s); break;
     case 32: e = w8 ? launch_split_batch<32, 8>(b, n_seq, max_splits, s) : launch_split_batch<32, 4>(b, n_seq, max_splits, s); break;
     case 64: e = w8 ? launch_split_batch<64, 8>(b, n_seq, max_splits, s) : launch_split_batch<64, 4>(b, n_seq, max_splits, s); break;
     case 128: e = w8 ? launch_split_batch<128, 8>(b, n_seq, max_splits, s) : launch_split_batch<128, 4>(b, n_seq, max_splits, s); break;

@@ -90,6 +90,7 @@ const Tuning &tuning() {
 // same number of wavefronts in flight; four are better when eight would leave three
 // quarters of the compute units without a workgroup (short contexts, ring layers).
 int choose_waves(const skv_layer *L, int n_pages_scan) {
+    if (L->g.P > 256) return 4; // one wavefront per SIMD: 512 registers each
     const size_t forced = tuning().forced_waves;
     if (forced == 4 || forced == 8) return (int)forced;
     const size_t kvh = (size_t)L->g.kv_heads;
@@ -136,7 +137,10 @@ int32_t check_window(const skv_layer *L, size_t window_start) {
     return SKV_OK;
 }
 
-bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L->g.P <= 256; }
+bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L->g.P <= 512; }
+// The fused pre-KV step and the LDS-shared prefill kernel are built up to head_dim 256; wider
+// heads take the separate norm/rotation launches and the 16-slot multi-query mode.
+bool wide_heads(const skv_layer *L) { return L->g.P > 256; }
 
 // Arguments of the matrix-core attention kernel for the layer's current length.
 void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, size_t window_start,
@@ -271,7 +275,7 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     // Chunks of at least 64 query slots take the kernel that shares each K/V page among 128
     // or 256 slots through LDS; shorter ones (speculative verify rows) the decode kernel's
     // multi-query mode, one workgroup per 16 slots.
-    const bool use_tiles = tuning().prefill_tiles && n_queries > 1 && n_queries * (size_t)g.gqa >= 64;
+    const bool use_tiles = tuning().prefill_tiles && n_queries > 1 && n_queries * (size_t)g.gqa >= 64 && g.P <= 256;
     if (n_queries > 1) {
         // split the context only while the query tiles alone leave compute units idle, and
         // keep the partials in the context's scratch
@@ -719,14 +723,13 @@ int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q
     if (!L || !q_dev || !k_dev || !v_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "prefill chunk: pointeur nul");
     if (n_rows == 0) return fail(SKV_ERR_DIMENSION, "attention batch cached shapes: seq == 0");
-    if (L->g.P > 256) return fail(SKV_ERR_CONFIG, "prefill sur cache: head_dim > 256 non supporté");
     if (L->len + n_rows > L->capacity)
         return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     const size_t kv_dim = skv_kv_dim(L), q_dim = (size_t)L->g.q_heads * L->g.head_dim;
     // Ring layers take the chunk in steps of at most the ring's rows (see ring_chunk).
     size_t step = std::min<size_t>(n_rows, 4096);
-    if (L->g.ring_rows > 0) step = std::min(step, (size_t)L->g.ring_rows);
+    if (L->g.ring_rows > 0) step = wide_heads(L) ? 1 : std::min(step, (size_t)L->g.ring_rows);
     const float *q = q_dev, *k = (const float *)k_dev, *v = (const float *)v_dev;
     float *out = out_dev;
     for (size_t done = 0; done < n_rows; done += step) {
@@ -989,7 +992,7 @@ static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope,
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     hipStream_t s = as_stream(stream);
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(L) || L->g.gqa > 16) {
+    if (!fused || !uses_flash(L) || wide_heads(L) || L->g.gqa > 16) {
         // the same step as separate launches: norm + rotation of q and k, append, attention, gate
         NormRopeArgs n{};
         n.x = q;

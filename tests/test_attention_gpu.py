@@ -63,7 +63,8 @@ def test_attention_decode_2pass_d128_matches_cpu(state, n):
 
 @pytest.mark.parametrize("dims", [(4, 2, 16), (4, 4, 64), (8, 1, 32), (6, 2, 96), (2, 1, 40),
                                   (32, 8, 128), (16, 8, 256), (32, 2, 128),
-                                  (40, 1, 64), (48, 2, 32)])   # the last two: more than 16 heads per group
+                                  (40, 1, 64), (48, 2, 32),    # these two: more than 16 heads per group
+                                  (8, 2, 512), (6, 1, 320), (34, 2, 512)])  # head_dim above 256: four-wavefront workgroups
 @pytest.mark.parametrize("n", [3, 100, 1500])
 def test_attention_decode_other_shapes(state, dims, n):
     run_attention_case(state, n, *dims)
@@ -264,6 +265,8 @@ def tiles_per_wavefront(request):
     ((6, 1, 40), 100, 100, 0),       # rows too short for 16-byte query loads, padded head_dim
     ((8, 1, 32), 33, 77, 0),         # head_dim 32, odd page count
     ((40, 1, 64), 10, 9, 0),         # GQA 40: 360 slots from 9 rows
+    ((8, 2, 512), 100, 70, 0),       # head_dim 512: the 16-slot multi-query mode, four wavefronts
+    ((4, 1, 320), 0, 33, 0),         # padded to 512
 ])
 def test_prefill_rows_match_per_row_oracle(state, tiles_per_wavefront, dims, start, chunk, window):
     """One launch == the reference's per-row loop (append, then cached_attention_one)."""
@@ -305,6 +308,24 @@ def test_prefill_rows_on_ring_layer(state, tiles_per_wavefront, window, chunks, 
     cache = oracle.LayerKvCache("bf16r")
     kv = state.full_attention_bf16(sum(chunks), q_heads, kv_heads, head_dim, window=window)
     for c in chunks:
+        q = rng.standard_normal((c, q_dim), dtype=np.float32)
+        k = rng.standard_normal((c, kv_dim), dtype=np.float32)
+        v = rng.standard_normal((c, kv_dim), dtype=np.float32)
+        got = kv.prefill_rows(q, k, v)
+        want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+        assert np.abs(got - want).max() <= 1e-4
+
+
+def test_prefill_rows_on_ring_layer_head_dim_512(state):
+    """Wider heads than the LDS-shared kernel is built for: a ring layer then advances row by
+    row through the decode kernel, with the same results."""
+    q_heads, kv_heads, head_dim, window = 4, 2, 512, 40
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(77)
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r")
+    kv = state.full_attention_bf16(120, q_heads, kv_heads, head_dim, window=window)
+    for c in (30, 50, 9):
         q = rng.standard_normal((c, q_dim), dtype=np.float32)
         k = rng.standard_normal((c, kv_dim), dtype=np.float32)
         v = rng.standard_normal((c, kv_dim), dtype=np.float32)
@@ -357,10 +378,19 @@ def test_flash_sdpa_off_uses_plain_kernel(state, env_flags, n, dims):
     assert np.abs(gpu - again).max() <= 2e-5      # the two device kernels agree with each other
 
 
-def test_plain_kernel_handles_head_dim_512_and_windows(state, env_flags):
-    """head_dim above 256 is served by the plain kernel whatever the flag says; the windowed
-    entry masks the rows before window_start there too (the reference's naive kernel is its
-    windowed path, src/decode_resident/attention.rs:780-786)."""
+@pytest.mark.parametrize("n", [9000, 40000])
+def test_attention_decode_head_dim_512_long_context(state, n):
+    """Global layers of Gemma-4-style models (global_head_dim 512, src/config/accessors.rs:118-123)
+    at lengths where the context is split."""
+    run_attention_case(state, n, 8, 2, 512)
+
+
+@pytest.mark.parametrize("flash", ["0", "1"])
+def test_head_dim_512_with_windows_on_both_kernels(state, env_flags, flash):
+    """head_dim 512 on the plain kernel (RETI_RUST_FLASH_SDPA=0) and on the matrix-core kernel;
+    the windowed entry masks the rows before window_start on both (the reference's naive kernel
+    is its windowed path, src/decode_resident/attention.rs:780-786)."""
+    env_flags(RETI_RUST_FLASH_SDPA=flash)
     q_heads, kv_heads, head_dim, n = 4, 2, 512, 90
     kv_dim = kv_heads * head_dim
     rng = np.random.default_rng(512)

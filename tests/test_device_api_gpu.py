@@ -79,6 +79,8 @@ def test_resident_device_append_then_read_same_stream(state):
     ((16, 8, 256), 64, 10, 200),     # ring layer: fills, wraps several times
     ((8, 2, 64), 48, 0, 120),        # ring from empty, window multiple of 16
     ((4, 2, 16), 20, 3, 70),         # window not a multiple of 16 (ring rounds up to 32 rows)
+    ((8, 2, 512), 0, 600, 20),       # head_dim 512, split-K
+    ((4, 2, 512), 32, 5, 60),        # head_dim 512 on a ring
 ])
 def test_fused_decode_steps_match_oracle(state, dims, window, start, steps):
     """Token by token: the fused append+attention step equals LayerKvCache::append +
@@ -157,6 +159,7 @@ def test_ring_layer_host_api(state):
     ((16, 8, 256), 64, [500, 0, 70, 63], 40),      # ring layers at different fill levels and wraps
     ((32, 8, 128), 0, [260, 2000], 20),            # two sequences, Qwen3-4B shape
     ((8, 2, 64), 0, list(range(100, 1900, 100)), 6),  # 18 sequences: more than one launch's worth
+    ((8, 2, 512), 0, [700, 20, 3000], 8),          # head_dim 512
 ])
 def test_decode_step_batch_matches_oracle(state, dims, window, starts, steps):
     """A batch of independent sequences through skv_decode_step_batch_device: every sequence

@@ -134,6 +134,7 @@ CASES = [
     ((4, 2, 16), 0, 3, 30, 4, 1.0e6, None, (True, True)),         # the reference's Gemma case: rope_dims = head_dim / 4
     ((8, 2, 64), 0, 0, 50, 64, 10000.0, 1.0, (False, False)),     # rotation only, from an empty cache
     ((6, 2, 96), 0, 20, 20, 32, 10000.0, None, (True, False)),    # q norm only, padded head_dim
+    ((8, 2, 512), 0, 300, 12, 128, 1.0e6, None, (True, True)),    # head_dim 512: norm/rotation as separate launches
 ]
 
 
