@@ -39,11 +39,11 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // several splits the (o, m, l) partials go to merge_rows_kernel.
 // ------------------------------------------------------------------------------------
 // Copies of PG pages (K tile then V tile each) of one kv head: memory -> registers -> LDS.
-template <int P, int PG>
-__device__ __forceinline__ void fetch_step(uint4 (&stage)[PG][(4 * (P / 32) * 32 + 511) / 512], const DecodeArgs &a,
+template <int P, int PG, int THREADS>
+__device__ __forceinline__ void fetch_step(uint4 (&stage)[PG][(2 * (P / 32) * 64 + THREADS - 1) / THREADS], const DecodeArgs &a,
                                            int pb0, int step, int n_it, int kvh, int tid) {
     constexpr int TILE_U4 = (P / 32) * 64;
-    constexpr int LOAD_U = (2 * TILE_U4 + 511) / 512;
+    constexpr int LOAD_U = (2 * TILE_U4 + THREADS - 1) / THREADS;
 #pragma unroll
     for (int pg = 0; pg < PG; ++pg) {
         // past the end: a page again, unused; always a page the layer holds
@@ -55,7 +55,7 @@ __device__ __forceinline__ void fetch_step(uint4 (&stage)[PG][(4 * (P / 32) * 32
 #pragma unroll
         for (int u = 0; u < LOAD_U; ++u) {
             // unconditional (a thread past the end re-reads the last unit and drops it)
-            const int i = min(tid + u * 512, 2 * TILE_U4 - 1);
+            const int i = min(tid + u * THREADS, 2 * TILE_U4 - 1);
             const uint4 *src = i < TILE_U4 ? kp + i : vp + (i - TILE_U4);
             stage[pg][u] = *src;
         }
@@ -65,19 +65,19 @@ __device__ __forceinline__ void fetch_step(uint4 (&stage)[PG][(4 * (P / 32) * 32
 // The K tiles are copied verbatim. The two V tiles of a pair are interleaved in 8-byte
 // halves, unit (kk, h, lane) = {page A's four keys, page B's four keys} of dim tile h, so
 // that one 16-byte read is the 32-key operand of the PV product as it stands.
-template <int P, int PG>
-__device__ __forceinline__ void store_step(const uint4 (&stage)[PG][(4 * (P / 32) * 32 + 511) / 512], uint4 *buf,
+template <int P, int PG, int THREADS>
+__device__ __forceinline__ void store_step(const uint4 (&stage)[PG][(2 * (P / 32) * 64 + THREADS - 1) / THREADS], uint4 *buf,
                                            int tid) {
     constexpr int TILE_U4 = (P / 32) * 64;
-    constexpr int LOAD_U = (2 * TILE_U4 + 511) / 512;
+    constexpr int LOAD_U = (2 * TILE_U4 + THREADS - 1) / THREADS;
     static_assert(PG % 2 == 0, "pages are consumed in pairs");
 #pragma unroll
     for (int pg = 0; pg < PG; ++pg) {
         uint4 *pair = buf + (pg >> 1) * 4 * TILE_U4;
 #pragma unroll
         for (int u = 0; u < LOAD_U; ++u) {
-            const int i = tid + u * 512;
-            if (2 * TILE_U4 < 512 && i >= 2 * TILE_U4) continue;
+            const int i = tid + u * THREADS;
+            if (2 * TILE_U4 < THREADS && i >= 2 * TILE_U4) continue;
             const uint4 x = stage[pg][u];
             if (i < TILE_U4) {
                 pair[(pg & 1) * TILE_U4 + i] = x;
@@ -93,10 +93,9 @@ __device__ __forceinline__ void store_step(const uint4 (&stage)[PG][(4 * (P / 32
 
 // PG: pages copied and consumed per barrier step (the copies of step i+1 are in flight while
 // step i is multiplied, so a step must hold about a memory latency's worth of work).
-template <int P, int TILES, int PG>
-__global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
-    constexpr int WAVES = 8;
-    constexpr int THREADS = 512;
+template <int P, int TILES, int PG, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) {
+    constexpr int THREADS = WAVES * 64;
     constexpr int KK = P / 32;
     constexpr int NT = P / 16;
     constexpr int TILE_U4 = KK * 64;                       // 16-byte units of one K (or V) tile
@@ -211,13 +210,13 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
     const int n_steps = (n_it + PG - 1) / PG;
     uint4 stage[PG][LOAD_U];
     // (a split without pages still reads one valid page, and writes empty partials below)
-    fetch_step<P, PG>(stage, a, pb0, 0, n_it, kvh, tid);
-    store_step<P, PG>(stage, kv_lds, tid);
+    fetch_step<P, PG, THREADS>(stage, a, pb0, 0, n_it, kvh, tid);
+    store_step<P, PG, THREADS>(stage, kv_lds, tid);
     __syncthreads();
 
     for (int step = 0; step < n_steps; ++step) {
       // unconditional: after the last step this re-reads its pages into the idle buffer
-      fetch_step<P, PG>(stage, a, pb0, min(step + 1, n_steps - 1), n_it, kvh, tid);
+      fetch_step<P, PG, THREADS>(stage, a, pb0, min(step + 1, n_steps - 1), n_it, kvh, tid);
       // Pages are consumed in pairs (A, B): the PV product then contracts over 32 keys with
       // the k index of lane group j, element e meaning key 4j+e of page A (e < 4) or key
       // 4j+e-4 of page B, which is exactly how the two S^T tiles and the two V tiles already
@@ -334,7 +333,7 @@ __global__ __launch_bounds__(512) void prefill_tile_kernel(DecodeArgs a) {
             }
         }
       }
-      store_step<P, PG>(stage, kv_lds + ((step + 1) & 1) * BUF_U4, tid);
+      store_step<P, PG, THREADS>(stage, kv_lds + ((step + 1) & 1) * BUF_U4, tid);
       __syncthreads();
     }
 
@@ -436,20 +435,23 @@ hipError_t launch_merge_rows(const DecodeArgs &a, hipStream_t s) {
 }
 
 // Query slots one workgroup of the kernel covers for a padded head_dim.
-int prefill_tile_slots(int P, bool two_tiles) { return two_tiles && prefill_two_tiles_possible(P) ? 256 : 128; }
+int prefill_tile_slots(int P, bool two_tiles) {
+    if (P > 256) return 64; // four wavefronts, one per SIMD (the accumulators and query halves are 256 registers)
+    return two_tiles && prefill_two_tiles_possible(P) ? 256 : 128;
+}
 // Two query tiles per wavefront need twice the accumulator and query registers: up to
 // head_dim 128.
 bool prefill_two_tiles_possible(int P) { return P <= 128; }
 
-template <int P, int TILES, int PG>
+template <int P, int TILES, int PG, int WAVES = 8>
 static hipError_t launch_tiles(const DecodeArgs &a, dim3 grid, hipStream_t s) {
     constexpr size_t lds = (size_t)2 * PG * 2 * (P / 32) * 64 * sizeof(uint4);
     static std::atomic<uint64_t> lds_ok{0}; // per instantiation
     {
-        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&prefill_tile_kernel<P, TILES, PG>), lds_ok);
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&prefill_tile_kernel<P, TILES, PG, WAVES>), lds_ok);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((prefill_tile_kernel<P, TILES, PG>), grid, dim3(512), lds, s, a);
+    hipLaunchKernelGGL((prefill_tile_kernel<P, TILES, PG, WAVES>), grid, dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
@@ -463,6 +465,7 @@ hipError_t launch_prefill_tiles(const DecodeArgs &a, hipStream_t s) {
     case 64: return two ? launch_tiles<64, 2, 8>(a, grid, s) : launch_tiles<64, 1, 8>(a, grid, s);
     case 128: return two ? launch_tiles<128, 2, 8>(a, grid, s) : launch_tiles<128, 1, 8>(a, grid, s);
     case 256: return launch_tiles<256, 1, 4>(a, grid, s);
+    case 512: return launch_tiles<512, 1, 2, 4>(a, grid, s);
     default: return hipErrorInvalidValue;
     }
 }

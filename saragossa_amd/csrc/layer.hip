@@ -138,8 +138,8 @@ int32_t check_window(const skv_layer *L, size_t window_start) {
 }
 
 bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L->g.P <= 512; }
-// The fused pre-KV step and the LDS-shared prefill kernel are built up to head_dim 256; wider
-// heads take the separate norm/rotation launches and the 16-slot multi-query mode.
+// The fused pre-KV step is built up to head_dim 256; wider heads take the separate
+// norm/rotation launches.
 bool wide_heads(const skv_layer *L) { return L->g.P > 256; }
 
 // Arguments of the matrix-core attention kernel for the layer's current length.
@@ -275,7 +275,7 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     // Chunks of at least 64 query slots take the kernel that shares each K/V page among 128
     // or 256 slots through LDS; shorter ones (speculative verify rows) the decode kernel's
     // multi-query mode, one workgroup per 16 slots.
-    const bool use_tiles = tuning().prefill_tiles && n_queries > 1 && n_queries * (size_t)g.gqa >= 64 && g.P <= 256;
+    const bool use_tiles = tuning().prefill_tiles && n_queries > 1 && n_queries * (size_t)g.gqa >= 64;
     if (n_queries > 1) {
         // split the context only while the query tiles alone leave compute units idle, and
         // keep the partials in the context's scratch
@@ -729,7 +729,7 @@ int32_t skv_prefill_chunk_device(skv_layer *L, skv_stream stream, const float *q
     const size_t kv_dim = skv_kv_dim(L), q_dim = (size_t)L->g.q_heads * L->g.head_dim;
     // Ring layers take the chunk in steps of at most the ring's rows (see ring_chunk).
     size_t step = std::min<size_t>(n_rows, 4096);
-    if (L->g.ring_rows > 0) step = wide_heads(L) ? 1 : std::min(step, (size_t)L->g.ring_rows);
+    if (L->g.ring_rows > 0) step = std::min(step, (size_t)L->g.ring_rows);
     const float *q = q_dev, *k = (const float *)k_dev, *v = (const float *)v_dev;
     float *out = out_dev;
     for (size_t done = 0; done < n_rows; done += step) {

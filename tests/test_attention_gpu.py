@@ -265,7 +265,8 @@ def tiles_per_wavefront(request):
     ((6, 1, 40), 100, 100, 0),       # rows too short for 16-byte query loads, padded head_dim
     ((8, 1, 32), 33, 77, 0),         # head_dim 32, odd page count
     ((40, 1, 64), 10, 9, 0),         # GQA 40: 360 slots from 9 rows
-    ((8, 2, 512), 100, 70, 0),       # head_dim 512: the 16-slot multi-query mode, four wavefronts
+    ((8, 2, 512), 100, 70, 0),       # head_dim 512: four wavefronts, 64 slots per workgroup
+    ((4, 1, 512), 700, 300, 0),      # head_dim 512, several workgroups and splits
     ((4, 1, 320), 0, 33, 0),         # padded to 512
 ])
 def test_prefill_rows_match_per_row_oracle(state, tiles_per_wavefront, dims, start, chunk, window):
@@ -317,8 +318,8 @@ def test_prefill_rows_on_ring_layer(state, tiles_per_wavefront, window, chunks, 
 
 
 def test_prefill_rows_on_ring_layer_head_dim_512(state):
-    """Wider heads than the LDS-shared kernel is built for: a ring layer then advances row by
-    row through the decode kernel, with the same results."""
+    """head_dim 512 on a ring layer: whole chunks in two phases around the append, on the
+    four-wavefront shape of the prefill kernel."""
     q_heads, kv_heads, head_dim, window = 4, 2, 512, 40
     kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
     rng = np.random.default_rng(77)
