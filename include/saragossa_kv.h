@@ -86,6 +86,12 @@ size_t skv_flag_prefill_chunk(void);              /* RETI_RUST_PREFILL_CHUNK (al
 void skv_flags_reload(void);
 /* window_start of a sliding layer (src/decoder/resident/types.rs:13-18); window 0 = none. */
 size_t skv_window_start(size_t position, size_t window);
+/* Rows a resident cache is created with: prefill_len + max_new_tokens + draft_headroom with
+ * checked additions (setup_resident_full_decode_with_slot, src/decoder/resident/setup.rs:322-329).
+ * Returns 1 and writes *capacity, or 0 when the sum overflows (the reference's
+ * "capacité KV résidente déborde"). A capacity of 0 means there is nothing to set up. */
+int32_t skv_resident_capacity(size_t prefill_len, size_t max_new_tokens, size_t draft_headroom,
+                              size_t *capacity);
 /* f32 -> bf16 bits, the reference's formula (src/decode_resident/utils.rs:55-60). Host helper. */
 uint16_t skv_f32_to_bf16_bits(float value);
 

@@ -182,6 +182,16 @@ size_t skv_window_start(size_t position, size_t window) {
     return position + 1 > window ? position + 1 - window : 0;
 }
 
+int32_t skv_resident_capacity(size_t prefill_len, size_t max_new_tokens, size_t draft_headroom,
+                              size_t *capacity) {
+    size_t a = 0, b = 0;
+    if (!capacity || __builtin_add_overflow(prefill_len, max_new_tokens, &a) ||
+        __builtin_add_overflow(a, draft_headroom, &b))
+        return 0;
+    *capacity = b;
+    return 1;
+}
+
 uint16_t skv_f32_to_bf16_bits(float value) {
     uint32_t bits;
     std::memcpy(&bits, &value, 4);

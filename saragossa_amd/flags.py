@@ -76,5 +76,14 @@ def window_start(position: int, window: int) -> int:
     return lib().skv_window_start(position, window)
 
 
+def resident_capacity(prefill_len: int, max_new_tokens: int, draft_headroom: int = 0):
+    """prefill + max_new + headroom, or None when the sum overflows
+    (src/decoder/resident/setup.rs:322-329)."""
+    import ctypes
+    out = ctypes.c_size_t(0)
+    ok = lib().skv_resident_capacity(prefill_len, max_new_tokens, draft_headroom, ctypes.byref(out))
+    return int(out.value) if ok else None
+
+
 def f32_to_bf16_bits(value: float) -> int:
     return lib().skv_f32_to_bf16_bits(value)

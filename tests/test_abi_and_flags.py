@@ -128,5 +128,12 @@ def test_integer_helpers_match_the_oracle():
         assert flags.sdpa_2pass_blocks(n) == oracle.sdpa_2pass_blocks(n)
     for pos, w in [(0, 0), (0, 4), (3, 4), (4, 4), (1023, 1024), (1024, 1024), (70000, 1024)]:
         assert flags.window_start(pos, w) == oracle.window_start(pos, w)
+    big = 2 ** 64 - 1
+    for a, b, c in [(0, 0, 0), (2048, 256, 0), (2048, 256, 4), (big, 0, 0), (big, 1, 0), (big - 5, 3, 3)]:
+        try:
+            want = oracle.resident_capacity(a, b, c)
+        except oracle.OracleError:
+            want = None
+        assert flags.resident_capacity(a, b, c) == want
     for x in [1.0039062, -0.33325195, 42.125, 0.0, 1e-40, 3.3895314e38]:
         assert flags.f32_to_bf16_bits(x) == int(oracle.f32_to_bf16_bits([x])[0])
