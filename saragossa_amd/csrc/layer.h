@@ -1,6 +1,9 @@
 // Host-side state of a context and of one layer's paged cache, shared by the entry points.
 #pragma once
 
+#include <map>
+#include <mutex>
+#include <utility>
 #include <vector>
 
 #include "skv_internal.h"
@@ -12,7 +15,24 @@ struct skv_ctx {
     hipStream_t stream = nullptr;
     void *mq_scratch = nullptr; // split-K partials of multi-query launches, grown on demand
     size_t mq_bytes = 0;
+    // Device buffers of destroyed layers, kept for the next layer that needs about as much:
+    // the stand-in for the arena DecodeResidentState leases its buffers from
+    // (src/decode_resident/arena.rs:116-211). A server creates and drops one cache per layer
+    // and request; without this every request pays hundreds of allocations and frees.
+    std::mutex arena_mu;
+    std::multimap<size_t, void *> arena_free; // by size in bytes
+    size_t arena_bytes = 0;                   // held in arena_free
+    size_t arena_cap = 0;                     // most it may hold (SKV_ARENA_MAX_MB, default 4096)
 };
+
+namespace skv {
+// A buffer of at least `bytes` from the context's arena (one whose size is within a quarter
+// above the need) or from hipMalloc; *got is its real size, to hand back with arena_put.
+hipError_t arena_get(skv_ctx *ctx, size_t bytes, void **ptr, size_t *got);
+// Returns a buffer to the arena, or frees it when the arena is full. The caller has made
+// sure the device no longer uses it.
+void arena_put(skv_ctx *ctx, void *ptr, size_t bytes);
+} // namespace skv
 
 struct skv_layer {
     skv_ctx *ctx = nullptr;
@@ -37,6 +57,7 @@ struct skv_layer {
     float *kv_stage = nullptr;  // [2*kv_dim]
     float *scores = nullptr;    // plain kernel: [q_heads][capacity], allocated on first use
     size_t scores_cap = 0;
+    std::vector<std::pair<void *, size_t>> leased; // buffers from the context's arena, with their sizes
 };
 
 // flags.cpp: generation counter of the cached runtime flags

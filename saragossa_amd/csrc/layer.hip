@@ -28,6 +28,39 @@ int32_t fail_hip(hipError_t e, const char *what) {
     return SKV_ERR_DEVICE;
 }
 
+hipError_t arena_get(skv_ctx *ctx, size_t bytes, void **ptr, size_t *got) {
+    *ptr = nullptr;
+    *got = 0;
+    if (bytes == 0) bytes = 256;
+    {
+        std::lock_guard<std::mutex> lk(ctx->arena_mu);
+        auto it = ctx->arena_free.lower_bound(bytes);
+        if (it != ctx->arena_free.end() && it->first <= bytes + bytes / 4) {
+            *ptr = it->second;
+            *got = it->first;
+            ctx->arena_bytes -= it->first;
+            ctx->arena_free.erase(it);
+            return hipSuccess;
+        }
+    }
+    const hipError_t e = hipMalloc(ptr, bytes);
+    if (e == hipSuccess) *got = bytes;
+    return e;
+}
+
+void arena_put(skv_ctx *ctx, void *ptr, size_t bytes) {
+    if (!ptr) return;
+    {
+        std::lock_guard<std::mutex> lk(ctx->arena_mu);
+        if (ctx->arena_bytes + bytes <= ctx->arena_cap) {
+            ctx->arena_free.emplace(bytes, ptr);
+            ctx->arena_bytes += bytes;
+            return;
+        }
+    }
+    (void)hipFree(ptr);
+}
+
 } // namespace skv
 
 using namespace skv;
@@ -365,6 +398,7 @@ int32_t skv_ctx_create(int32_t device, skv_ctx **out) try {
     skv_ctx *c = new skv_ctx();
     c->device = device;
     c->stream = nullptr;
+    c->arena_cap = env_usize("SKV_ARENA_MAX_MB", 4096) << 20;
     *out = c;
     return SKV_OK;
 } catch (...) {
@@ -376,6 +410,7 @@ void skv_ctx_destroy(skv_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
     if (ctx->mq_scratch) (void)hipFree(ctx->mq_scratch);
+    for (auto &kv : ctx->arena_free) (void)hipFree(kv.second);
     delete ctx;
 }
 
@@ -392,10 +427,8 @@ void skv_layer_destroy(skv_layer *L) {
     if (!L) return;
     (void)hipSetDevice(L->ctx->device);
     (void)hipDeviceSynchronize();
-    for (void *p : {(void *)L->k_pool, (void *)L->v_pool, (void *)L->table_dev, (void *)L->part_o,
-                    (void *)L->part_m, (void *)L->part_l, (void *)L->q_stage,
-                    (void *)L->out_stage, (void *)L->kv_stage, (void *)L->scores})
-        if (p) (void)hipFree(p);
+    for (auto &b : L->leased) arena_put(L->ctx, b.first, b.second);
+    if (L->scores) (void)hipFree(L->scores);
     delete L;
 }
 
@@ -443,7 +476,10 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
 
     hipError_t e = hipSuccess;
     auto alloc = [&](void **p, size_t bytes) {
-        if (e == hipSuccess) e = hipMalloc(p, bytes);
+        if (e != hipSuccess) return;
+        size_t got = 0;
+        e = arena_get(ctx, bytes, p, &got);
+        if (e == hipSuccess) L->leased.emplace_back(*p, got);
     };
     alloc((void **)&L->k_pool, pool_bytes);
     alloc((void **)&L->v_pool, pool_bytes);

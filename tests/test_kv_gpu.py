@@ -170,3 +170,32 @@ def test_bf16_rounding_special_values(state):
     want = oracle.f32_to_bf16_bits(data)
     assert np.array_equal(gk, want)
     assert np.array_equal(gv, want)
+
+
+def test_buffers_of_a_destroyed_layer_are_reused_clean(state):
+    """The context keeps the device buffers of destroyed layers for the next layer of about
+    the same size (the arena of DecodeResidentState, src/decode_resident/arena.rs:116-211). A
+    layer that inherits them must not see what the previous owner left: its padded dims and
+    unwritten rows are zero again (head_dim 96 is padded to 128, so stale values there would
+    enter every score)."""
+    import oracle
+    rng = np.random.default_rng(123)
+    first = state.full_attention_bf16(512, 8, 2, 128)
+    first.seed(rng.standard_normal((512, 256), dtype=np.float32) * 50,
+               rng.standard_normal((512, 256), dtype=np.float32) * 50, 512)
+    first.close()
+    # same pool bytes (512 rows x 2 heads x 128 padded dims), other logical shape
+    kv = state.full_attention_bf16(512, 6, 2, 96)
+    n, kv_dim = 300, 2 * 96
+    keys = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    values = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    kv.seed(keys, values, n)
+    q = rng.standard_normal(6 * 96, dtype=np.float32)
+    lay = oracle.layout(6, 2, 96)
+    cache = oracle.LayerKvCache("bf16r")
+    cache.append_batch(keys, values, lay)
+    want = oracle.cached_attention_one(q, cache, lay)
+    assert np.abs(kv.attention_decode(q) - want).max() <= 1e-4
+    gk, gv = kv.read_rows_f32()
+    assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
+    kv.close()
