@@ -271,6 +271,7 @@ GATED = [
     ((16, 2, 256), 0, 3, 30, 64, 1.0e7),      # short cache: the split kernel applies the gate itself
     ((8, 4, 64), 32, 5, 80, 64, 10000.0),     # ring layer
     ((6, 2, 96), 0, 40, 10, 48, 10000.0),     # padded head_dim
+    ((4, 2, 512), 0, 100, 8, 128, 1.0e6),     # head_dim 512: every stage a launch of its own
 ]
 
 
