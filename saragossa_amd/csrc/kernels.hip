@@ -116,6 +116,18 @@ hipError_t launch_append(const AppendArgs &a, hipStream_t s) {
     return hipGetLastError();
 }
 
+// Identity block table of a fresh layer, written on the device (no host-to-device copy).
+__global__ __launch_bounds__(256) void iota_kernel(int32_t *dst, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = i;
+}
+
+hipError_t launch_iota(int32_t *dst, int n, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(iota_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, dst, n);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------------------------------
 // gather: tiles -> row-major bf16 rows [n_rows, kv_dim], through the block table.
 // ------------------------------------------------------------------------------------

@@ -496,9 +496,7 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     if (e == hipSuccess) e = hipMemsetAsync(L->v_pool, 0, pool_bytes, ctx->stream);
     L->table.resize(L->n_pages);
     for (int i = 0; i < L->n_pages; ++i) L->table[i] = i;
-    if (e == hipSuccess)
-        e = hipMemcpyAsync(L->table_dev, L->table.data(), (size_t)L->n_pages * sizeof(int32_t),
-                           hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = launch_iota(L->table_dev, L->n_pages, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
         skv_layer_destroy(L);

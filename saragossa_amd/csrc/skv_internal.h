@@ -177,6 +177,7 @@ struct GateArgs {
     int heads, head_dim, gate_head_stride;
 };
 hipError_t launch_gate(const GateArgs &a, hipStream_t s);
+hipError_t launch_iota(int32_t *dst, int n, hipStream_t s);
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s);
 
 // Raises a kernel's dynamic LDS limit to the 160 KiB of a gfx950 compute unit, once per
