@@ -199,3 +199,48 @@ def test_buffers_of_a_destroyed_layer_are_reused_clean(state):
     gk, gv = kv.read_rows_f32()
     assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
     kv.close()
+
+
+def test_a_context_gives_all_device_memory_back():
+    """Handles own their device memory exactly once (src/decoder.rs:434-446): after a context
+    of its own has created and dropped layers, snapshots, a rotation table and a hot cache,
+    and has itself been destroyed (which empties its arena), the device has as much free
+    memory as before. (A first context goes through the same motions beforehand, so that what
+    the runtime keeps for itself after first use is not counted.)"""
+    torch = pytest.importorskip("torch")
+
+    def lifetime(rounds):
+        st = skv.DecodeResidentState(0)
+        rng = np.random.default_rng(9)
+        for _ in range(rounds):
+            layers = [st.full_attention_bf16(4096, 32, 8, 128, window=(1024 if i == 1 else 0)) for i in range(4)]
+            for kv in layers:
+                kv.seed(rng.standard_normal((600, 1024), dtype=np.float32),
+                        rng.standard_normal((600, 1024), dtype=np.float32), 600)
+            q = rng.standard_normal(32 * 128, dtype=np.float32)
+            layers[0].attention_decode(q)
+            layers[0].prefill_rows(rng.standard_normal((40, 4096), dtype=np.float32),
+                                   rng.standard_normal((40, 1024), dtype=np.float32),
+                                   rng.standard_normal((40, 1024), dtype=np.float32))
+            snap = skv.snapshot_blocks(st, [layers[0], layers[2]], [0, 5, 7])
+            copy = snap.clone()
+            rope = st.rope_table(4096, 128, 1.0e6)
+            hot = skv.HotCache(st, 16, 64, 32, layers)
+            root = skv.BlockHash.root()
+            h = skv.BlockHash.chain(root, list(range(16)))
+            assert hot.remember_prefix_block(root, h, 16, layers)
+            hot.close()
+            rope.close()
+            copy.close()
+            snap.close()
+            for kv in layers:
+                kv.close()
+        st.close()
+        torch.cuda.synchronize()
+
+    lifetime(1)
+    torch.cuda.empty_cache()
+    free0, _ = torch.cuda.mem_get_info()
+    lifetime(3)
+    free1, _ = torch.cuda.mem_get_info()
+    assert free0 - free1 <= 16 << 20, (free0, free1)
