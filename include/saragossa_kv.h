@@ -47,7 +47,10 @@ typedef struct skv_hot skv_hot;
  * The *_device entry points only queue work on that stream: they neither wait for the
  * device nor switch devices, so the stream must belong to the context's device and that
  * device must be current on the calling thread (the *_host entry points and the create /
- * destroy calls make it current themselves). Host-side bookkeeping (len, ring position)
+ * destroy calls make it current themselves). Two exceptions allocate, after a device
+ * synchronisation: a chunked-prefill call whose split partials need more scratch than any
+ * call before it on the context (the buffer only grows), and the first attention call of a
+ * layer on the plain kernel (RETI_RUST_FLASH_SDPA=0), which creates its score buffer. Host-side bookkeeping (len, ring position)
  * advances when the call returns, before the device has run the work, exactly like the
  * reference's encode-time `len += 1` (src/decode_resident/attention.rs:993); buffers handed
  * to a *_device call must stay valid until the stream has passed that work. */
