@@ -588,6 +588,43 @@ def main() -> int:
     kern_ms = sorted(e0.elapsed_time(e1) / layers_n for e0, e1 in evs)
     kern_avg_us = sum(kern_ms) / len(kern_ms) * 1e3
     kern_med_us = kern_ms[len(kern_ms) // 2] * 1e3
+
+    # ---- what the hardware allows at this size: a launch per layer that only fetches the same
+    # K and V pages (same grid, same access pattern, nothing computed, nothing merged), and an
+    # empty launch; timed the same way, ten launches between two events
+    ceiling = None
+    if B == 1:
+        def timed_launches(fn, per_pair):
+            pairs = []
+            for _ in range(max(args.steps // 2, 20)):
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                pairs.append((e0, e1))
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) * 1e3 / per_pair for a, b in pairs[3:])
+            return ts[len(ts) // 2]
+
+        def read_all():
+            for kv in layers:
+                kv.encode_probe_read_pages(stream)
+
+        def empty_all():
+            for _ in layers:
+                state.encode_probe_empty_launch(stream)
+
+        read_us = timed_launches(read_all, layers_n)
+        empty_us = timed_launches(empty_all, layers_n)
+        kv_bytes = sum(2 * min(kv.len(), kv.window() or kv.len()) * kv_dim * 2 for kv in layers) // layers_n
+        ceiling = {"read_only_launch_us": round(read_us, 2),
+                   "read_only_gbps": round(kv_bytes / read_us / 1e3, 1),
+                   "read_only_frac_of_peak": round(kv_bytes / read_us / 1e3 / HBM_PEAK_GBPS, 4),
+                   "empty_launch_us": round(empty_us, 2),
+                   "attention_vs_read_only": round(read_us / kern_avg_us, 3),
+                   "note": "a launch per layer that only fetches the cached K/V pages with the decode "
+                           "kernel's grid and access pattern (no products, no partials, no merge)"}
     # the dominant launch is a layer of the first group; with mixed groups the event pairs span
     # all layers, so bytes are summed over the layers and divided by the same time
     late = total_steps + args.steps // 2
@@ -674,6 +711,8 @@ def main() -> int:
                      "p10_launch_us": round(kern_ms[len(kern_ms) // 10] * 1e3, 2),
                      "p90_launch_us": round(kern_ms[len(kern_ms) * 9 // 10] * 1e3, 2)},
     }
+    if ceiling is not None:
+        result["ceiling"] = ceiling
     if restore is not None:
         result["restore"] = restore
     if recurrent is not None:

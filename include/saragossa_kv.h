@@ -102,6 +102,11 @@ uint16_t skv_f32_to_bf16_bits(float value);
 
 /* DecodeResidentState::new(device) (src/decoder/resident/setup.rs:237, 675). */
 int32_t skv_ctx_create(int32_t device, skv_ctx **out);
+/* Waits for the device, gives back the device memory the context itself holds and ends the
+ * caller's use of `ctx`. Layers, rope tables, snapshots and hot caches made from it stay valid
+ * until their own destroy call (the order of the destroy calls is free, as with finalisers of a
+ * garbage-collected binding); making new objects from a destroyed context is an error of the
+ * caller. */
 void skv_ctx_destroy(skv_ctx *ctx);
 /* Blocks until everything queued on the context's own stream has finished. */
 int32_t skv_ctx_synchronize(skv_ctx *ctx);
@@ -282,6 +287,16 @@ int32_t skv_read_rows(skv_layer *layer, size_t first, size_t n, uint16_t *k_out,
 /* Same gather, device to device, async on `stream`. */
 int32_t skv_gather_device(skv_layer *layer, skv_stream stream, size_t first, size_t n,
                           void *k_dst_dev, void *v_dst_dev);
+
+/* ---- measurement aids (no counterpart in the reference; used by bench.py) ---- */
+
+/* Reads every K and V page of the layer's first `len` rows once, through the block table, with
+ * the decode kernel's grid and access pattern (256 workgroups of 8 wavefronts by default, 16-byte
+ * non-temporal loads of whole tiles) and does nothing with them: what a launch that only
+ * had to fetch the cache would cost. Async on `stream`. */
+int32_t skv_probe_read_pages_device(skv_layer *layer, skv_stream stream);
+/* An empty kernel with the decode launch's shape: the cost of a launch alone. */
+int32_t skv_probe_empty_launch_device(skv_ctx *ctx, skv_stream stream);
 
 /* ---- block snapshots: snapshot/copy/restore_prompt_state_metal ------------- */
 

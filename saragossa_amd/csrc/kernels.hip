@@ -129,6 +129,55 @@ hipError_t launch_iota(int32_t *dst, int n, hipStream_t s) {
 }
 
 // ------------------------------------------------------------------------------------
+// Measurement aids: a launch that only fetches the cache the way the decode kernel does
+// (grid (splits, kv heads), eight wavefronts, each walking its share of the pages and loading
+// the K and V tile of its kv head with 16-byte non-temporal loads, 1 KiB per instruction), and
+// an empty launch of the same shape.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(512) void probe_read_kernel(ProbeArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int split = blockIdx.x, kvh = blockIdx.y;
+    const int pb0 = (int)(((long)split * a.n_pages) / a.splits);
+    const int pb1 = (int)(((long)(split + 1) * a.n_pages) / a.splits);
+    const int units = a.g.tile_elems >> 3; // 16-byte units of one tile
+    uint32_t acc = 0;
+    for (int pb = pb0 + wave; pb < pb1; pb += 8) {
+        const int page = __builtin_amdgcn_readfirstlane(a.table[pb]);
+        const long tile = (long)page * a.g.page_elems + (long)kvh * a.g.tile_elems;
+        typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+        const u32x4_t *kp = reinterpret_cast<const u32x4_t *>(a.k_pool + tile);
+        const u32x4_t *vp = reinterpret_cast<const u32x4_t *>(a.v_pool + tile);
+        for (int u = lane; u < units; u += 64 * 8) {
+            u32x4_t k[8], v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int at = min(u + i * 64, units - 1);
+                k[i] = __builtin_nontemporal_load(kp + at);
+                v[i] = __builtin_nontemporal_load(vp + at);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc ^= k[i].x ^ k[i].w ^ v[i].y ^ v[i].z;
+        }
+    }
+    if (acc == 0x9e3779b9u && a.sink) a.sink[0] = acc; // keeps the loads alive
+}
+
+__global__ __launch_bounds__(512) void probe_empty_kernel(uint32_t *sink) {
+    if (sink && threadIdx.x == 0xffff) sink[0] = 1;
+}
+
+hipError_t launch_probe_read(const ProbeArgs &a, hipStream_t s) {
+    if (a.n_pages <= 0 || a.splits <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)a.splits, (unsigned)a.g.kv_heads), dim3(512), 0, s, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_probe_empty(hipStream_t s) {
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(256), dim3(512), 0, s, (uint32_t *)nullptr);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------
 // gather: tiles -> row-major bf16 rows [n_rows, kv_dim], through the block table.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void gather_kernel(GatherArgs a) {

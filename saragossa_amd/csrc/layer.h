@@ -1,6 +1,7 @@
 // Host-side state of a context and of one layer's paged cache, shared by the entry points.
 #pragma once
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -23,6 +24,12 @@ struct skv_ctx {
     std::multimap<size_t, void *> arena_free; // by size in bytes
     size_t arena_bytes = 0;                   // held in arena_free
     size_t arena_cap = 0;                     // most it may hold (SKV_ARENA_MAX_MB, default 4096)
+    // One reference for the owner plus one per layer, rope table, snapshot and hot cache made
+    // from the context: skv_ctx_destroy gives the context's device memory back and drops the
+    // owner's reference, the struct itself goes with the last object that points at it, so a
+    // binding whose finalisers run in any order never touches freed memory.
+    std::atomic<int> refs{1};
+    bool closed = false; // after skv_ctx_destroy: arena_put frees instead of keeping
 };
 
 namespace skv {
@@ -32,10 +39,33 @@ hipError_t arena_get(skv_ctx *ctx, size_t bytes, void **ptr, size_t *got);
 // Returns a buffer to the arena, or frees it when the arena is full. The caller has made
 // sure the device no longer uses it.
 void arena_put(skv_ctx *ctx, void *ptr, size_t bytes);
+void ctx_release(skv_ctx *ctx);
+
+// The context pointer of an object made from a context; holds one of its references.
+class CtxRef {
+  public:
+    CtxRef() = default;
+    CtxRef(const CtxRef &o) { *this = o.p_; }
+    CtxRef &operator=(const CtxRef &o) { return *this = o.p_; }
+    ~CtxRef() {
+        if (p_) ctx_release(p_);
+    }
+    CtxRef &operator=(skv_ctx *c) {
+        if (c) c->refs.fetch_add(1, std::memory_order_relaxed);
+        if (p_) ctx_release(p_);
+        p_ = c;
+        return *this;
+    }
+    skv_ctx *operator->() const { return p_; }
+    operator skv_ctx *() const { return p_; }
+
+  private:
+    skv_ctx *p_ = nullptr;
+};
 } // namespace skv
 
 struct skv_layer {
-    skv_ctx *ctx = nullptr;
+    skv::CtxRef ctx;
     Geom g{};
     size_t capacity = 0;
     size_t len = 0;

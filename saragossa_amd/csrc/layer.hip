@@ -52,13 +52,35 @@ void arena_put(skv_ctx *ctx, void *ptr, size_t bytes) {
     if (!ptr) return;
     {
         std::lock_guard<std::mutex> lk(ctx->arena_mu);
-        if (ctx->arena_bytes + bytes <= ctx->arena_cap) {
+        if (!ctx->closed && ctx->arena_bytes + bytes <= ctx->arena_cap) {
             ctx->arena_free.emplace(bytes, ptr);
             ctx->arena_bytes += bytes;
             return;
         }
     }
     (void)hipFree(ptr);
+}
+
+// Frees what the context holds on the device; the caller has synchronised the device.
+static void ctx_drain(skv_ctx *ctx) {
+    std::lock_guard<std::mutex> lk(ctx->arena_mu);
+    if (ctx->mq_scratch) (void)hipFree(ctx->mq_scratch);
+    ctx->mq_scratch = nullptr;
+    ctx->mq_bytes = 0;
+    for (auto &kv : ctx->arena_free) (void)hipFree(kv.second);
+    ctx->arena_free.clear();
+    ctx->arena_bytes = 0;
+}
+
+void ctx_release(skv_ctx *ctx) {
+    if (ctx->refs.fetch_sub(1, std::memory_order_acq_rel) != 1) return;
+    // a layer that outlived skv_ctx_destroy may have grown the multi-query scratch again
+    if (ctx->mq_scratch) {
+        (void)hipSetDevice(ctx->device);
+        (void)hipDeviceSynchronize();
+        ctx_drain(ctx);
+    }
+    delete ctx;
 }
 
 } // namespace skv
@@ -409,9 +431,12 @@ void skv_ctx_destroy(skv_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
-    if (ctx->mq_scratch) (void)hipFree(ctx->mq_scratch);
-    for (auto &kv : ctx->arena_free) (void)hipFree(kv.second);
-    delete ctx;
+    {
+        std::lock_guard<std::mutex> lk(ctx->arena_mu);
+        ctx->closed = true;
+    }
+    ctx_drain(ctx);
+    ctx_release(ctx);
 }
 
 int32_t skv_ctx_synchronize(skv_ctx *ctx) try {
@@ -829,7 +854,7 @@ int32_t skv_prefill_chunk_host(skv_layer *L, const float *q, const float *k, con
 // ---- the step before the cache: per-head RMSNorm + rotation --------------------------
 
 struct skv_rope {
-    skv_ctx *ctx = nullptr;
+    CtxRef ctx;
     float *table = nullptr; // [max_positions][rope_dims/2][2]
     size_t max_positions = 0;
     size_t rope_dims = 0;
@@ -1270,6 +1295,32 @@ int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uin
     if (rc) return rc;
     if (e != hipSuccess) return fail_hip(e, "read_rows: copie device→hôte");
     if (e2 != hipSuccess) return fail_hip(e2, "read_rows: synchronisation");
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+// ---- measurement aids ---------------------------------------------------------------------
+int32_t skv_probe_read_pages_device(skv_layer *L, skv_stream stream) try {
+    if (!L) return fail(SKV_ERR_DEVICE, "probe: pointeur nul");
+    if (L->len == 0) return fail(SKV_ERR_DIMENSION, "probe: cache vide");
+    ProbeArgs a{};
+    a.k_pool = L->k_pool;
+    a.v_pool = L->v_pool;
+    a.table = L->table_dev;
+    a.sink = nullptr;
+    a.n_pages = (int)std::min<size_t>((L->len + 15) / 16, (size_t)L->n_pages);
+    a.splits = (int)std::max<size_t>(std::min<size_t>(decode_target_wgs() / (size_t)L->g.kv_heads, (size_t)a.n_pages), 1);
+    a.g = L->g;
+    SKV_HIP(launch_probe_read(a, as_stream(stream)));
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_probe_empty_launch_device(skv_ctx *ctx, skv_stream stream) try {
+    if (!ctx) return fail(SKV_ERR_DEVICE, "probe: ctx nul");
+    SKV_HIP(launch_probe_empty(as_stream(stream)));
     return SKV_OK;
 } catch (...) {
     return skv::fail_exception();

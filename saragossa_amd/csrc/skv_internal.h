@@ -178,6 +178,19 @@ struct GateArgs {
 };
 hipError_t launch_gate(const GateArgs &a, hipStream_t s);
 hipError_t launch_iota(int32_t *dst, int n, hipStream_t s);
+
+// Measurement aids (a read-only walk of the cache with the decode kernel's pattern; an empty launch).
+struct ProbeArgs {
+    const uint16_t *k_pool;
+    const uint16_t *v_pool;
+    const int32_t *table;
+    uint32_t *sink;
+    int n_pages;
+    int splits;
+    Geom g;
+};
+hipError_t launch_probe_read(const ProbeArgs &a, hipStream_t s);
+hipError_t launch_probe_empty(hipStream_t s);
 hipError_t launch_norm_rope(const NormRopeArgs &a, hipStream_t s);
 
 // Raises a kernel's dynamic LDS limit to the 160 KiB of a gfx950 compute unit, once per

@@ -245,7 +245,7 @@ static int32_t check_layers(skv_ctx *ctx, skv_layer *const *layers, size_t n_lay
 using namespace skv;
 
 struct skv_snapshot {
-    skv_ctx *ctx = nullptr;
+    CtxRef ctx;
     uint8_t *base = nullptr;
     size_t bytes = 0;
     // block snapshots
@@ -265,7 +265,7 @@ struct HotEntry {
 };
 
 struct skv_hot {
-    skv_ctx *ctx = nullptr;
+    CtxRef ctx;
     PrefixIndex *index = nullptr;
     SlotLayout layout;
     size_t pages_per_block = 0;

@@ -85,6 +85,10 @@ class DecodeResidentState:
         check(self._l.skv_attn_gate_device(self._h, stream, ctx_ptr, gate_ptr, gate_head_stride,
                                            heads, head_dim, out_ptr))
 
+    def encode_probe_empty_launch(self, stream) -> None:
+        """Measurement aid: an empty kernel with the decode launch's shape."""
+        check(self._l.skv_probe_empty_launch_device(self._h, stream))
+
     def rope_table(self, max_positions, rope_dims, theta, position_scale=1.0, frequency_dim=0,
                    style=0) -> "RopeTable":
         return RopeTable(self, max_positions, rope_dims, theta, position_scale, frequency_dim, style)
@@ -229,6 +233,11 @@ class FullAttentionState:
 
     def encode_attention_decode_windowed(self, stream, q_ptr, out_ptr, window_start) -> None:
         check(self._l.skv_attention_device(self._h, stream, q_ptr, out_ptr, window_start))
+
+    def encode_probe_read_pages(self, stream) -> None:
+        """Measurement aid: a launch that only fetches the cached K and V pages, with the
+        decode kernel's grid and access pattern."""
+        check(self._l.skv_probe_read_pages_device(self._h, stream))
 
     def encode_decode_step(self, stream, k_ptr, k_off, v_ptr, v_off, q_ptr, out_ptr) -> None:
         check(self._l.skv_decode_step_device(self._h, stream, k_ptr, k_off, v_ptr, v_off, q_ptr,

@@ -314,3 +314,30 @@ def test_attention_launches_replay_correctly_from_a_hip_graph(state):
         torch.cuda.synchronize()
         for o, e in zip(outs, eager):
             assert torch.equal(o, e), f"replay {replay}"
+
+
+def test_measurement_probes_leave_the_cache_untouched(state):
+    # the read-only and empty launches that the benchmark times beside the attention launch:
+    # they run on full and ring layers at ragged lengths and change nothing
+    rng = np.random.default_rng(31)
+    for (q_heads, kv_heads, head_dim), window, n in (((16, 2, 256), None, 1000), ((8, 2, 128), 64, 333),
+                                                     ((8, 8, 64), None, 1), ((4, 1, 512), None, 47)):
+        kv_dim = kv_heads * head_dim
+        kv = state.full_attention_bf16(n + 4, q_heads, kv_heads, head_dim, window=window or 0)
+        with pytest.raises(skv.DimensionError):
+            kv.encode_probe_read_pages(_stream())
+        kv.seed(rng.standard_normal((n, kv_dim), dtype=np.float32),
+                rng.standard_normal((n, kv_dim), dtype=np.float32), n)
+        first = max(0, n - window) if window else 0
+        before = kv.read_rows(first)
+        q = rng.standard_normal(q_heads * head_dim, dtype=np.float32)
+        attend = (lambda: kv.attention_decode_windowed(q, first)) if window else (lambda: kv.attention_decode(q))
+        want = attend()
+        for _ in range(3):
+            kv.encode_probe_read_pages(_stream())
+            state.encode_probe_empty_launch(_stream())
+        torch.cuda.synchronize()
+        after = kv.read_rows(first)
+        assert np.array_equal(before[0], after[0]) and np.array_equal(before[1], after[1])
+        assert np.array_equal(attend(), want)
+        kv.close()

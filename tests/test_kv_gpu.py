@@ -244,3 +244,41 @@ def test_a_context_gives_all_device_memory_back():
     lifetime(3)
     free1, _ = torch.cuda.mem_get_info()
     assert free0 - free1 <= 16 << 20, (free0, free1)
+
+
+def test_objects_may_outlive_their_context():
+    """Finalisers of a garbage-collected binding run in any order: a layer, a rope table, a
+    snapshot and a hot cache stay usable after skv_ctx_destroy and are destroyed afterwards,
+    and all device memory still comes back."""
+    torch = pytest.importorskip("torch")
+
+    def lifetime():
+        st = skv.DecodeResidentState(0)
+        rng = np.random.default_rng(10)
+        layers = [st.full_attention_bf16(2048, 32, 8, 128) for _ in range(3)]
+        keys = rng.standard_normal((300, 1024), dtype=np.float32)
+        values = rng.standard_normal((300, 1024), dtype=np.float32)
+        for kv in layers:
+            kv.seed(keys, values, 300)
+        snap = skv.snapshot_blocks(st, layers[:2], [0, 3])
+        rope = st.rope_table(1024, 128, 1.0e6)
+        hot = skv.HotCache(st, 16, 32, 32, layers)
+        q = rng.standard_normal(32 * 128, dtype=np.float32)
+        want = layers[0].attention_decode(q)
+        copy = snap.clone()
+        layers[2].close()  # into the arena, which the next line empties
+        st.close()
+        assert np.array_equal(layers[0].attention_decode(q), want)
+        layers[1].append_row(keys[0], values[0])
+        assert layers[1].len() == 301
+        for obj in (layers[0], hot, copy, rope, snap, layers[1]):
+            obj.close()
+        torch.cuda.synchronize()
+
+    lifetime()
+    torch.cuda.empty_cache()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        lifetime()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free0 - free1 <= 16 << 20, (free0, free1)
