@@ -4,6 +4,15 @@ import sys
 import numpy as np
 import pytest
 
+# torch ships its own copy of the HIP runtime. A process can initialise only one: whichever
+# of torch and libsaragossa_kv.so is loaded first decides which copy both then use, and torch
+# finds no GPU on a runtime that is not its own. The GPU tests use torch tensors as device
+# memory, so torch goes first here.
+try:
+    import torch  # noqa: F401
+except ImportError:
+    pass
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
