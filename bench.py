@@ -51,12 +51,15 @@ WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {2: 70135 * 1024}
 
 
+ELEM_BYTES = 2  # bytes of a cached K or V element in the decode leg: 2 (bf16) or 4 (--element f32)
+
+
 def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> int:
-    """Bytes one layer's decode step has to move: K and V once (bf16), q in and ctx out
-    (f32), the block table, and the appended row when the append is counted."""
-    b = 2 * rows * kv_dim * 2 + 2 * q_dim * 4 + (rows + 15) // 16 * 4
+    """Bytes one layer's decode step has to move: K and V once (in the cache's element), q in
+    and ctx out (f32), the block table, and the appended row when the append is counted."""
+    b = 2 * rows * kv_dim * ELEM_BYTES + 2 * q_dim * 4 + (rows + 15) // 16 * 4
     if with_append:
-        b += 2 * kv_dim * 2
+        b += 2 * kv_dim * ELEM_BYTES
     return b
 
 
@@ -448,6 +451,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=0, help="override the cached rows")
     ap.add_argument("--batch", type=int, default=1,
                     help="independent sequences decoded together (configs[4] also asks for 4)")
+    ap.add_argument("--element", choices=["bf16", "f32"], default="bf16",
+                    help="element of the decode leg's caches (f32 is the reference's choice for greedy decoding)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-restore", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -467,6 +472,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the KV path has no CPU fallback", file=sys.stderr)
         return 2
+    global ELEM_BYTES
+    ELEM_BYTES = 4 if args.element == "f32" else 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.config == 3:
@@ -499,7 +506,9 @@ def main() -> int:
     for n, _, _, _, rows, window in groups:
         for _ in range(n):
             for _ in range(B):   # every sequence owns its pages and its block table
-                kv = state.full_attention_bf16(rows + 2 * total_steps + 8, qh, kvh, hd, window=window)
+                kv = state.full_attention_with_element(rows + 2 * total_steps + 8, qh, kvh, hd,
+                                                       skv.DTYPE_F32 if args.element == "f32" else skv.DTYPE_BF16,
+                                                       window)
                 kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
                 fill = min(rows, window) if window else rows   # a ring only keeps its window
                 k = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
@@ -617,7 +626,7 @@ def main() -> int:
 
         read_us = timed_launches(read_all, layers_n)
         empty_us = timed_launches(empty_all, layers_n)
-        kv_bytes = sum(2 * min(kv.len(), kv.window() or kv.len()) * kv_dim * 2 for kv in layers) // layers_n
+        kv_bytes = sum(2 * min(kv.len(), kv.window() or kv.len()) * kv_dim * ELEM_BYTES for kv in layers) // layers_n
         ceiling = {"read_only_launch_us": round(read_us, 2),
                    "read_only_gbps": round(kv_bytes / read_us / 1e3, 1),
                    "read_only_frac_of_peak": round(kv_bytes / read_us / 1e3 / HBM_PEAK_GBPS, 4),
@@ -691,21 +700,23 @@ def main() -> int:
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": args.element,
         "data": "synthetic",
-        "config": {"workload": (wl["name"] % ctx_rows) + ", bf16 KV in 16-token pages, batch %d, "
-                               "1 token per sequence per step" % B,
+        "config": {"workload": (wl["name"] % ctx_rows) + ", %s KV in 16-token pages, batch %d, "
+                               "1 token per sequence per step" % (args.element, B),
                    "context": ctx_rows, "layers": layers_n, "page_rows": 16, "batch": B},
         "tok_per_s": round(1e6 / us_per_token, 1),
         "hbm_gbps": round(step_bytes / (step_us * 1e-6) / 1e9, 1),
         "hbm_frac": round(step_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-        "roofline": {"bound": "hbm", "kernel": ("decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
+        "roofline": {"bound": "hbm", "kernel": ("f32_split_kernel<%d> + decode_merge_kernel (one attention launch per "
+                                                "sequence, average over the layers)" if args.element == "f32" else
+                                                "decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
                                                 "average over the layers)" if B == 1 else
                                                 "decode_split_batch_kernel<%d,8> + decode_merge_batch_kernel (one launch pair "
                                                 "per layer covers the batch, average over the layers)")
                                                % (128 if hd <= 128 else 256),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context and B == 1 else None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context and B == 1 and args.element == "bf16" else None,
                      "bytes_per_launch": launch_bytes,
                      "avg_launch_us": round(kern_avg_us, 2), "median_launch_us": round(kern_med_us, 2),
                      "p10_launch_us": round(kern_ms[len(kern_ms) // 10] * 1e3, 2),

@@ -32,7 +32,7 @@ extern "C" {
 #define SKV_ERR_CONFIG 2    /* InferError::Config: zero dimension, bad GQA ratio, unsupported option */
 #define SKV_ERR_DEVICE 3    /* InferError::Metal: device/runtime failure, null pointer, wrong element */
 
-#define SKV_DTYPE_F32 0  /* GpuElement::F32 — not built; skv_layer_create rejects it */
+#define SKV_DTYPE_F32 0  /* GpuElement::F32: rows kept as they arrive (head_dim up to 256) */
 #define SKV_DTYPE_BF16 1 /* GpuElement::Bf16 */
 
 #define SKV_PAGE_ROWS 16
@@ -116,7 +116,10 @@ int32_t skv_ctx_synchronize(skv_ctx *ctx);
 /* DecodeResidentState::full_attention_with_element (src/decode_resident/attention.rs:56-108).
  * Rejects a zero dimension and q_heads % kv_heads != 0 with SKV_ERR_CONFIG.
  * `window` > 0 makes the layer a ring buffer that keeps the last `window` rows
- * (rounded up to whole pages); 0 keeps all `capacity` rows in pages. */
+ * (rounded up to whole pages); 0 keeps all `capacity` rows in pages.
+ * `dtype` is what the pages hold: SKV_DTYPE_BF16 (rows rounded to nearest even at append,
+ * head_dim up to 512) or SKV_DTYPE_F32 (rows verbatim, head_dim up to 256; pages twice the
+ * bytes). Every entry point below serves both; where they differ it says so. */
 int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
                          size_t head_dim, int32_t dtype, size_t window, skv_layer **out);
 /* full_attention(capacity, q_heads, kv_heads, head_dim, sampled) (attention.rs:26-45):
@@ -282,9 +285,12 @@ int32_t skv_decode_step_layers_device(skv_layer *const *layers, size_t n_layers,
 
 /* Reads logical rows [first, first+n) through the block table as bf16 bits,
  * row-major [n, kv_dim]: the stand-in for reading keys()/values() back
- * (tests.rs:423-428, 469-476). Synchronous. */
+ * (tests.rs:423-428, 469-476). Synchronous. bf16 layers only (SKV_ERR_CONFIG on an f32 one). */
 int32_t skv_read_rows(skv_layer *layer, size_t first, size_t n, uint16_t *k_out, uint16_t *v_out);
-/* Same gather, device to device, async on `stream`. */
+/* The same rows as f32, for layers of either element type (bf16 rows widen exactly). */
+int32_t skv_read_rows_f32(skv_layer *layer, size_t first, size_t n, float *k_out, float *v_out);
+/* Same gather, device to device, async on `stream`; the destination rows have the layer's
+ * element type (bf16 bits or f32). */
 int32_t skv_gather_device(skv_layer *layer, skv_stream stream, size_t first, size_t n,
                           void *k_dst_dev, void *v_dst_dev);
 

@@ -103,6 +103,7 @@ SIGNATURES = {
     "skv_decode_step_batch_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_decode_step_layers_device": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "skv_read_rows": (_i32, [_vp, _sz, _sz, _vp, _vp]),
+    "skv_read_rows_f32": (_i32, [_vp, _sz, _sz, _vp, _vp]),
     "skv_gather_device": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp]),
     "skv_snapshot_blocks": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, C.POINTER(_vp)]),
     "skv_snapshot_clone": (_i32, [_vp, _vp, _vp, C.POINTER(_vp)]),

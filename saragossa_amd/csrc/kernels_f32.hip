@@ -1,0 +1,340 @@
+// gfx950 kernels of the KV hot path, part 4: the f32 storage mode of the cache
+// (KvElement::F32, src/decode_resident/attention.rs:26-45; the reference's default for greedy
+// decoding, src/decode_resident/utils.rs:202-210). Same pages, block table, ring and split
+// partials as the bf16 mode; the tiles hold f32 and the products run on the f32 matrix
+// instruction (v_mfma_f32_16x16x4_f32), which has the operand layout of the bf16 kernels'
+// 16x16 tiles with a contraction of 4 per instruction.
+//
+// Tile layouts (one tile = 16 rows x P dims of one kv head, P * 16 floats), chosen so that a
+// wavefront's operand fetch is one contiguous KiB and a lane's 16-byte load is four
+// consecutive contraction steps:
+//   K: float4 unit (m, j, r) = dims 16m + 4j .. +3 of row r, at unit index m * 64 + j * 16 + r
+//   V: float4 unit (c, jj, dd) = rows 4jj .. 4jj+3 of dim 16c + dd, at unit index c * 64 + jj * 16 + dd
+#include "skv_internal.h"
+
+namespace skv {
+
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+
+__host__ __device__ inline int k_index_f32(int r, int d) {
+    return (((d >> 4) * 64 + ((d >> 2) & 3) * 16 + r) << 2) + (d & 3);
+}
+__host__ __device__ inline int v_index_f32(int r, int d) {
+    return (((d >> 4) * 64 + (r >> 2) * 16 + (d & 15)) << 2) + (r & 3);
+}
+
+namespace {
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+} // namespace
+
+// ------------------------------------------------------------------------------------
+// append: rows [n_rows, kv_dim] f32 -> tiles, verbatim. One thread per (row, kv head, four
+// dims): a 16-byte K store and four 4-byte V stores.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void append_f32_kernel(AppendArgs a) {
+    const Geom g = a.g;
+    const int groups = (g.head_dim + 3) >> 2;
+    const long per_row = (long)g.kv_heads * groups;
+    const long total = per_row * a.n_rows;
+    const int kv_dim = g.kv_heads * g.head_dim;
+    float *k_pool = reinterpret_cast<float *>(a.k_pool);
+    float *v_pool = reinterpret_cast<float *>(a.v_pool);
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const int row = (int)(t / per_row);
+        const int rem = (int)(t - (long)row * per_row);
+        const int kvh = rem / groups;
+        const int d0 = (rem - kvh * groups) * 4;
+        const long slot = slot_of(a.first_pos + row, g.ring_rows);
+        const int page = a.table[slot >> 4];
+        const int r = (int)(slot & 15);
+        // tile_elems and page_elems count 16-bit units: two per float
+        const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
+        const float *ks = a.k_src + (long)row * kv_dim + kvh * g.head_dim + d0;
+        const float *vs = a.v_src + (long)row * kv_dim + kvh * g.head_dim + d0;
+        float4_t kq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) kq[e] = d0 + e < g.head_dim ? ks[e] : 0.0f;
+        *reinterpret_cast<float4_t *>(k_pool + tile + k_index_f32(r, d0)) = kq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (d0 + e < g.head_dim) v_pool[tile + v_index_f32(r, d0 + e)] = vs[e];
+    }
+}
+
+hipError_t launch_append_f32(const AppendArgs &a, hipStream_t s) {
+    const long total = (long)a.g.kv_heads * ((a.g.head_dim + 3) >> 2) * a.n_rows;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65535 * 4) blocks = 65535 * 4;
+    hipLaunchKernelGGL(append_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+// gather: tiles -> row-major f32 rows [n_rows, kv_dim], through the block table.
+__global__ __launch_bounds__(256) void gather_f32_kernel(GatherArgs a) {
+    const Geom g = a.g;
+    const int kv_dim = g.kv_heads * g.head_dim;
+    const long total = (long)kv_dim * a.n_rows;
+    const float *k_pool = reinterpret_cast<const float *>(a.k_pool);
+    const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
+    float *k_dst = reinterpret_cast<float *>(a.k_dst);
+    float *v_dst = reinterpret_cast<float *>(a.v_dst);
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const int row = (int)(t / kv_dim);
+        const int col = (int)(t - (long)row * kv_dim);
+        const int kvh = col / g.head_dim;
+        const int d = col - kvh * g.head_dim;
+        const long slot = slot_of(a.first_pos + row, g.ring_rows);
+        const int page = a.table[slot >> 4];
+        const int r = (int)(slot & 15);
+        const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
+        if (k_dst) k_dst[t] = k_pool[tile + k_index_f32(r, d)];
+        if (v_dst) v_dst[t] = v_pool[tile + v_index_f32(r, d)];
+    }
+}
+
+hipError_t launch_gather_f32(const GatherArgs &a, hipStream_t s) {
+    const long total = (long)a.g.kv_heads * a.g.head_dim * a.n_rows;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65535 * 4) blocks = 65535 * 4;
+    hipLaunchKernelGGL(gather_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------
+// Attention over the f32 cache, decode and chunked prefill alike (cached_attention_one and
+// cached_attention_prefill_rows, src/decoder/attention_ops.rs:976-1046): query slot
+// (i, g) = query row i, head g of the kv head's group, attends positions up to
+// min(q_pos0 + i, limit_cap) through the layer's window.
+//
+// grid (splits, kv heads, tiles of 16 query slots); a workgroup is four wavefronts that take
+// the pages of its split in turn. A wavefront holds the 16 slots' queries (pre-scaled by
+// log2(e)/sqrt(head_dim)) and its own (o, m, l) in registers and streams K and V tiles straight
+// from memory into the matrix operands: S^T = K . Q^T (16 keys x 16 slots), one online-softmax
+// step in base 2 per page, O^T += V^T . P^T with the probabilities taken from the very
+// registers the scores arrived in (contraction step k of lane group jj is key 4jj + k, which
+// is where the score tile keeps it). The four wavefronts' states meet in LDS at the end; the
+// workgroup writes the context (one split) or its (o, m, l) partial in the layout of the
+// bf16 kernels, for the same merge kernels.
+// ------------------------------------------------------------------------------------
+template <int P>
+__global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
+    constexpr int NT = P / 16;
+    extern __shared__ __attribute__((aligned(16))) float4_t xch[]; // [4 wavefronts][NT][64] o | [4][16] m | [4][16] l
+    const Geom g = a.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15; // slot column of the tiles; key row of the K operand; dim of the V operand
+    const int j = lane >> 4; // lane group
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int G = g.gqa;
+    const int n_slots = a.n_queries * G;
+    const int slot0 = blockIdx.z * 16;
+    const int s_last = min(slot0 + 15, n_slots - 1);
+    const int my_slot = min(slot0 + n, n_slots - 1);
+
+    auto pos_of = [&](int slot) { return a.q_pos0 + slot / G; };
+    auto limit_of = [&](int slot) { return min(pos_of(slot), a.limit_cap); };
+    auto ws_of = [&](int slot) { return a.window > 0 ? max(a.window_start, pos_of(slot) + 1 - a.window) : a.window_start; };
+    const int my_limit = limit_of(my_slot), my_ws = ws_of(my_slot);
+    const int t_ws_lo = ws_of(slot0), t_ws_hi = ws_of(s_last);
+    const int t_lim_lo = limit_of(slot0), t_lim_hi = limit_of(s_last);
+
+    // pages any slot of the tile can see, divided among the splits, then among the wavefronts
+    const int page_lo = g.ring_rows > 0 ? 0 : t_ws_lo >> 4;
+    const int page_hi = g.ring_rows > 0 ? a.n_pages : (t_lim_hi >> 4) + 1;
+    const unsigned span = (unsigned)max(page_hi - page_lo, 0);
+    const int pb0 = page_lo + (int)(((unsigned)split * span) / (unsigned)a.splits);
+    const int pb1 = page_lo + (int)(((unsigned)(split + 1) * span) / (unsigned)a.splits);
+
+    // queries: lane (slot n, group j) holds dims 16m + 4j .. +3 of every block m
+    float4_t qv[NT];
+    {
+        const float *qrow = a.q + ((long)(my_slot / G) * g.q_heads + kvh * G + my_slot % G) * g.head_dim;
+        // all loads first, unconditional from clamped addresses (one round trip); dims past
+        // head_dim are zeroed afterwards
+        if (a.q_vec) {
+#pragma unroll
+            for (int m = 0; m < NT; ++m)
+                qv[m] = *reinterpret_cast<const float4_t *>(qrow + min(m * 16 + j * 4, g.head_dim - 4));
+        } else {
+#pragma unroll
+            for (int m = 0; m < NT; ++m) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) qv[m][e] = qrow[min(m * 16 + j * 4 + e, g.head_dim - 1)];
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < NT; ++m) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) qv[m][e] = m * 16 + j * 4 + e < g.head_dim ? qv[m][e] * a.qscale : 0.0f;
+        }
+    }
+    float4_t o[NT];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    const float *k_pool = reinterpret_cast<const float *>(a.k_pool);
+    const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
+    const int last_page = a.page_first + a.n_pages - 1;
+    // (every page of [page_lo, page_hi) is visible to some slot of the tile)
+    auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
+        const int page = a.table[min(pb, last_page)];
+        const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
+        const float4_t *kt = reinterpret_cast<const float4_t *>(k_pool + tile);
+        const float4_t *vt = reinterpret_cast<const float4_t *>(v_pool + tile);
+#pragma unroll
+        for (int m = 0; m < NT; ++m) kq[m] = kt[m * 64 + lane];
+#pragma unroll
+        for (int c = 0; c < NT; ++c) vq[c] = vt[c * 64 + lane];
+    };
+    auto consume = [&](int pb, const float4_t (&kq)[NT], const float4_t (&vq)[NT]) {
+        const int slot_a = pb * 16; // first cache slot of the page
+        // S^T = K . Q^T: two accumulators so that consecutive products do not wait for each other
+        float4_t s0 = float4_t{0.f, 0.f, 0.f, 0.f}, s1 = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < NT; ++m) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][0], qv[m][0], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][1], qv[m][1], s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][2], qv[m][2], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][3], qv[m][3], s1, 0, 0, 0);
+        }
+        float sv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sv[e] = s0[e] + s1[e];
+        const bool interior = g.ring_rows == 0 && slot_a >= t_ws_hi && slot_a + 15 <= t_lim_lo;
+        if (!interior) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int slot = slot_a + j * 4 + e; // this lane's key e
+                int pos = slot;
+                if (g.ring_rows > 0) pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+                sv[e] = (pos >= my_ws && pos <= my_limit) ? sv[e] : -INFINITY;
+            }
+        }
+        float m_blk = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+        m_blk = rows_max(m_blk);
+        const float m_new = fmaxf(m_run, m_blk);
+        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        float pv[4];
+        float psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            pv[e] = fast_exp2(sv[e] - m_safe);
+            psum += pv[e];
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) o[c] *= alpha;
+        }
+        // O^T += V^T . P^T, contraction step outermost: consecutive products use different accumulators
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq[c][k], pv[k], o[c], 0, 0, 0);
+        }
+    };
+    // The page after the one being multiplied is already on its way into a second set of
+    // registers: without that every wavefront of the device loads, then multiplies, in step,
+    // and memory idles half the time.
+    float4_t k_a[NT], v_a[NT], k_b[NT], v_b[NT];
+    int pb = pb0 + wave;
+    if (pb < pb1) fetch(pb, k_a, v_a);
+    while (pb < pb1) {
+        if (pb + 4 < pb1) fetch(pb + 4, k_b, v_b);
+        consume(pb, k_a, v_a);
+        pb += 4;
+        if (pb >= pb1) break;
+        if (pb + 4 < pb1) fetch(pb + 4, k_a, v_a);
+        consume(pb, k_b, v_b);
+        pb += 4;
+    }
+
+    // ---- the four wavefronts' states meet in LDS ------------------------------------------
+    float *xm = reinterpret_cast<float *>(xch + 4 * NT * 64);
+    float *xl = xm + 64;
+    const float l_mine = rows_sum(l_run);
+#pragma unroll
+    for (int c = 0; c < NT; ++c) xch[(wave * NT + c) * 64 + lane] = o[c];
+    if (j == 0) {
+        xm[wave * 16 + n] = m_run;
+        xl[wave * 16 + n] = l_mine;
+    }
+    __syncthreads();
+    float mw[4], lw[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        mw[w] = xm[w * 16 + n];
+        lw[w] = xl[w * 16 + n];
+        mx = fmaxf(mx, mw[w]);
+    }
+    const float m_safe = mx == -INFINITY ? 0.0f : mx;
+    float l = 0.0f;
+    float sc[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        sc[w] = fast_exp2(mw[w] - m_safe);
+        l += sc[w] * lw[w];
+    }
+    const int slot = slot0 + n;
+    if (slot >= n_slots) return;
+    float *dst;
+    float scale = 1.0f;
+    if (a.splits_total == 1) {
+        scale = 1.0f / l;
+        dst = a.out + ((long)(slot / G) * g.q_heads + kvh * G + slot % G) * g.head_dim;
+    } else {
+        const long pidx = ((long)kvh * a.splits_total + a.split_base + split) * n_slots + slot;
+        dst = a.part_o + pidx * g.head_dim;
+        if (j == 0 && wave == 0) {
+            a.part_m[pidx] = mx;
+            a.part_l[pidx] = l;
+        }
+    }
+    // wavefront w finishes the dim tiles c = w, w + 4, ...
+    for (int c = wave; c < NT; c += 4) {
+        float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) acc += xch[(w * NT + c) * 64 + lane] * sc[w];
+        acc *= scale;
+        const int col = c * 16 + j * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (col + i < g.head_dim) dst[col + i] = acc[i];
+    }
+}
+
+template <int P>
+static hipError_t launch_f32(const DecodeArgs &a, dim3 grid, hipStream_t s) {
+    constexpr size_t lds = (size_t)4 * (P / 16) * 64 * sizeof(float4_t) + 2 * 64 * sizeof(float);
+    static std::atomic<uint64_t> lds_ok{0}; // per instantiation
+    {
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_split_kernel<P>), lds_ok);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((f32_split_kernel<P>), grid, dim3(256), lds, s, a);
+    return hipGetLastError();
+}
+
+// The split launch of an f32 layer; the caller merges (launch_merge for one query row,
+// launch_merge_rows for a chunk) when splits_total > 1.
+hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
+    if (a.k_new || a.pre) return hipErrorInvalidValue; // no fused append or pre-KV step in this mode
+    const int n_slots = a.n_queries * a.g.gqa;
+    dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
+    switch (a.g.P) {
+    case 32: return launch_f32<32>(a, grid, s);
+    case 64: return launch_f32<64>(a, grid, s);
+    case 128: return launch_f32<128>(a, grid, s);
+    case 256: return launch_f32<256>(a, grid, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+} // namespace skv

@@ -286,6 +286,28 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     int32_t rc = check_window(L, window_start);
     if (rc) return rc;
     const Geom &g = L->g;
+    if (g.f32) {
+        // the f32 storage mode has one attention kernel (no plain variant, no fused append or
+        // pre-KV step): 16 query slots per workgroup, the context split while that leaves
+        // compute units idle
+        if (k_new || v_new || pre) return fail(SKV_ERR_CONFIG, "KV f32: étape fusionnée non construite");
+        DecodeArgs a{};
+        fill_decode_args(L, q_dev, out_dev, window_start, nullptr, nullptr, n_queries, decode_target_wgs(), a);
+        if (attn_scalar > 0.0f) a.qscale = (1.0f / std::sqrt(attn_scalar)) * 1.4426950408889634f;
+        if (n_queries > 1) {
+            const size_t tiles = (n_queries * (size_t)g.gqa + 15) / 16 * (size_t)g.kv_heads;
+            const size_t want = std::max<size_t>(2 * decode_target_wgs() / tiles, 1);
+            a.splits = (int)std::min<size_t>((size_t)a.splits, want);
+            a.splits_total = a.splits;
+            if (a.splits > 1) {
+                int32_t rc2 = multi_query_partials(L, (size_t)a.splits, n_queries, a);
+                if (rc2) return rc2;
+            }
+        }
+        SKV_HIP(launch_f32_split(a, s));
+        if (a.splits > 1) SKV_HIP(n_queries > 1 ? launch_merge_rows(a, s) : launch_merge(a, s));
+        return SKV_OK;
+    }
     const bool use_flash = uses_flash(L) || n_queries > 1;
     if (!use_flash) {
         const size_t need = (size_t)g.q_heads * L->capacity;
@@ -382,6 +404,13 @@ int32_t encode_append(skv_layer *L, hipStream_t s, const float *k_dev, const flo
         a.first_pos += (long)skip;
         a.n_rows = L->g.ring_rows;
     }
+    if (L->g.f32) {
+        SKV_HIP(launch_append_f32(a, s));
+        L->len += n_rows;
+        if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
+            L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
+        return SKV_OK;
+    }
     // whole groups of four rows at positions that are multiples of 4 write V in 16-byte units
     if (a.n_rows >= 8) {
         a.by_page = 1;
@@ -466,10 +495,12 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     if (q_heads % kv_heads != 0)
         return fail(SKV_ERR_CONFIG, "GQA invalide: q_heads=" + std::to_string(q_heads) +
                                         " non multiple de kv_heads=" + std::to_string(kv_heads));
-    if (dtype != SKV_DTYPE_BF16)
-        return fail(SKV_ERR_CONFIG, "KV f32 non construit dans cette bibliothèque: bf16 uniquement");
+    if (dtype != SKV_DTYPE_BF16 && dtype != SKV_DTYPE_F32)
+        return fail(SKV_ERR_CONFIG, "élément KV inconnu: " + std::to_string(dtype));
+    const bool f32 = dtype == SKV_DTYPE_F32;
     const int P = padded_head_dim(head_dim);
     if (P == 0) return fail(SKV_ERR_CONFIG, "head_dim > 512 non supporté");
+    if (f32 && P > 256) return fail(SKV_ERR_CONFIG, "KV f32: head_dim > 256 non supporté");
     if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096)
         return fail(SKV_ERR_CONFIG, "capacité KV déborde");
     SKV_HIP(hipSetDevice(ctx->device));
@@ -484,7 +515,8 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     g.head_dim = (int)head_dim;
     g.P = P;
     g.gqa = (int)(q_heads / kv_heads);
-    g.tile_elems = P * 16;
+    g.f32 = f32 ? 1 : 0;
+    g.tile_elems = P * 16 * (f32 ? 2 : 1);
     g.page_elems = (int)kv_heads * g.tile_elems;
     size_t rows = capacity;
     if (window > 0) {
@@ -572,7 +604,7 @@ size_t skv_kv_heads(const skv_layer *L) { return L ? (size_t)L->g.kv_heads : 0; 
 size_t skv_head_dim(const skv_layer *L) { return L ? (size_t)L->g.head_dim : 0; }
 size_t skv_window(const skv_layer *L) { return L ? L->window : 0; }
 size_t skv_logical_byte_len(const skv_layer *L) {
-    return L ? L->capacity * (size_t)L->g.kv_heads * L->g.head_dim * 2 : 0;
+    return L ? L->capacity * (size_t)L->g.kv_heads * L->g.head_dim * (L->g.f32 ? 4 : 2) : 0;
 }
 
 int32_t skv_truncate(skv_layer *L, size_t len) try {
@@ -697,7 +729,7 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
     if (!L || !k_dev || !v_dev || !q_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step: pointeur nul");
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(L)) {
+    if (!fused || !uses_flash(L) || L->g.f32) {
         int32_t rc = skv_append_device(L, stream, k_dev, k_off, v_dev, v_off);
         if (rc) return rc;
         const size_t ws = skv_window_start(L->len - 1, L->window);
@@ -731,11 +763,12 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
                           size_t c, float *out) {
     const Geom &g = L->g;
     const size_t base = L->len;
-    const bool two = prefill_two_tiles(g, L->n_pages);
-    const size_t per_wg = (size_t)prefill_tile_slots(g.P, two);
+    const bool two = !g.f32 && prefill_two_tiles(g, L->n_pages);
+    const size_t per_wg = g.f32 ? 16 : (size_t)prefill_tile_slots(g.P, two);
     const size_t tiles = (c * (size_t)g.gqa + per_wg - 1) / per_wg * (size_t)g.kv_heads;
+    auto launch_chunk = [&](const DecodeArgs &a) { return g.f32 ? launch_f32_split(a, s) : launch_prefill_tiles(a, s); };
     auto splits_for = [&](int n_pages) {
-        size_t want = std::max<size_t>(tuning().prefill_wgs / tiles, 1);
+        size_t want = std::max<size_t>((g.f32 ? 2 : 1) * tuning().prefill_wgs / tiles, 1);
         want = std::min<size_t>(want, std::max<size_t>((size_t)n_pages / 8, 1));
         return (int)std::min<size_t>(want, tuning().prefill_max_splits);
     };
@@ -757,7 +790,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
         a1.splits_total = total;
         int32_t rc = multi_query_partials(L, (size_t)total, c, a1);
         if (rc) return rc;
-        SKV_HIP(launch_prefill_tiles(a1, s));
+        SKV_HIP(launch_chunk(a1));
     }
     int32_t rc = encode_append(L, s, k, v, c);
     if (rc) return rc;
@@ -771,7 +804,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
         rc = multi_query_partials(L, (size_t)total, c, a3);
         if (rc) return rc;
     }
-    SKV_HIP(launch_prefill_tiles(a3, s));
+    SKV_HIP(launch_chunk(a3));
     if (total > 1) SKV_HIP(launch_merge_rows(a3, s));
     return SKV_OK;
 }
@@ -1051,7 +1084,7 @@ static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope,
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     hipStream_t s = as_stream(stream);
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(L) || wide_heads(L) || L->g.gqa > 16) {
+    if (!fused || !uses_flash(L) || wide_heads(L) || L->g.gqa > 16 || L->g.f32) {
         // the same step as separate launches: norm + rotation of q and k, append, attention, gate
         NormRopeArgs n{};
         n.x = q;
@@ -1173,7 +1206,8 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
             return fail(SKV_ERR_DEVICE, "decode_step_batch: pointeur nul (séquence " + std::to_string(i) + ")");
         const Geom &g = L->g, &g0 = seqs[0]->g;
         if (g.q_heads != g0.q_heads || g.kv_heads != g0.kv_heads || g.head_dim != g0.head_dim ||
-            g.ring_rows != g0.ring_rows || L->window != seqs[0]->window || L->ctx != seqs[0]->ctx)
+            g.ring_rows != g0.ring_rows || g.f32 != g0.f32 || L->window != seqs[0]->window ||
+            L->ctx != seqs[0]->ctx)
             return fail(SKV_ERR_DIMENSION, "decode_step_batch: la séquence " + std::to_string(i) +
                                                " n'a pas la géométrie de la séquence 0");
         for (size_t j = 0; j < i; ++j)
@@ -1185,7 +1219,7 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
                                                " atteinte (overflow), séquence " + std::to_string(i));
     }
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(seqs[0]) || seqs[0]->g.gqa > 16 || n_seq == 1) {
+    if (!fused || !uses_flash(seqs[0]) || seqs[0]->g.gqa > 16 || n_seq == 1 || seqs[0]->g.f32) {
         for (size_t i = 0; i < n_seq; ++i) {
             int32_t rc = skv_decode_step_device(seqs[i], stream, k_dev[i], 0, v_dev[i], 0, q_dev[i], out_dev[i]);
             if (rc) return rc;
@@ -1269,7 +1303,47 @@ int32_t skv_gather_device(skv_layer *L, skv_stream stream, size_t first, size_t 
     a.first_pos = (long)first;
     a.n_rows = (int)n;
     a.g = L->g;
-    SKV_HIP(launch_gather(a, as_stream(stream)));
+    SKV_HIP(L->g.f32 ? launch_gather_f32(a, as_stream(stream)) : launch_gather(a, as_stream(stream)));
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+// Rows of either storage mode as f32 (bf16 rows widened: exact).
+int32_t skv_read_rows_f32(skv_layer *L, size_t first, size_t n, float *k_out, float *v_out) try {
+    if (!L) return fail(SKV_ERR_DEVICE, "read_rows: pointeur nul");
+    int32_t rc = check_rows(L, first, n);
+    if (rc) return rc;
+    if (n == 0) return SKV_OK;
+    const size_t elems = n * skv_kv_dim(L);
+    if (!L->g.f32) {
+        std::vector<uint16_t> kb(k_out ? elems : 0), vb(v_out ? elems : 0);
+        rc = skv_read_rows(L, first, n, k_out ? kb.data() : nullptr, v_out ? vb.data() : nullptr);
+        if (rc) return rc;
+        auto widen = [](uint16_t b) {
+            const uint32_t u = (uint32_t)b << 16;
+            float f;
+            std::memcpy(&f, &u, sizeof f);
+            return f;
+        };
+        for (size_t i = 0; i < kb.size(); ++i) k_out[i] = widen(kb[i]);
+        for (size_t i = 0; i < vb.size(); ++i) v_out[i] = widen(vb[i]);
+        return SKV_OK;
+    }
+    SKV_HIP(hipSetDevice(L->ctx->device));
+    float *tmp = nullptr;
+    SKV_HIP(hipMalloc((void **)&tmp, 2 * elems * sizeof(float)));
+    hipStream_t s = L->ctx->stream;
+    float *kd = tmp, *vd = tmp + elems;
+    rc = skv_gather_device(L, s, first, n, k_out ? kd : nullptr, v_out ? vd : nullptr);
+    hipError_t e = hipSuccess;
+    if (!rc && k_out) e = hipMemcpyAsync(k_out, kd, elems * sizeof(float), hipMemcpyDeviceToHost, s);
+    if (!rc && e == hipSuccess && v_out) e = hipMemcpyAsync(v_out, vd, elems * sizeof(float), hipMemcpyDeviceToHost, s);
+    hipError_t e2 = hipStreamSynchronize(s);
+    (void)hipFree(tmp);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail_hip(e, "read_rows: copie device→hôte");
+    if (e2 != hipSuccess) return fail_hip(e2, "read_rows: synchronisation");
     return SKV_OK;
 } catch (...) {
     return skv::fail_exception();
@@ -1277,6 +1351,7 @@ int32_t skv_gather_device(skv_layer *L, skv_stream stream, size_t first, size_t 
 
 int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uint16_t *v_out) try {
     if (!L) return fail(SKV_ERR_DEVICE, "read_rows: pointeur nul");
+    if (L->g.f32) return fail(SKV_ERR_CONFIG, "read_rows: cache f32, lire avec skv_read_rows_f32");
     int32_t rc = check_rows(L, first, n);
     if (rc) return rc;
     if (n == 0) return SKV_OK;

@@ -58,9 +58,10 @@ struct Geom {
     int head_dim;
     int P;          // padded head dim
     int gqa;        // q_heads / kv_heads
-    int tile_elems; // P * 16: one (page, kv head) tile
+    int tile_elems; // one (page, kv head) tile in 16-bit units: P * 16 (bf16), P * 32 (f32)
     int page_elems; // kv_heads * tile_elems
     int ring_rows;  // 0 = full cache; else rows kept by the ring (multiple of 16)
+    int f32;        // 1 = the tiles hold f32 (kernels_f32.hip), 0 = bf16
 };
 
 __host__ __device__ inline int k_index(int P, int r, int d) {
@@ -312,6 +313,11 @@ struct NaiveArgs {
 // ---- launchers (kernels.hip) ------------------------------------------------------
 hipError_t launch_append(const AppendArgs &a, hipStream_t s);
 hipError_t launch_gather(const GatherArgs &a, hipStream_t s);
+// f32 storage mode: rows in and out (k_dst / v_dst of GatherArgs then point at f32 rows), and
+// the split launch for one query row or a chunk (the caller merges as for bf16)
+hipError_t launch_append_f32(const AppendArgs &a, hipStream_t s);
+hipError_t launch_gather_f32(const GatherArgs &a, hipStream_t s);
+hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s);
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s);
 hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s);
 hipError_t launch_merge(const DecodeArgs &a, hipStream_t s);        // split-K partials -> context

@@ -11,7 +11,7 @@ import ctypes as C
 
 import numpy as np
 
-from ._lib import DTYPE_BF16, check, lib
+from ._lib import DTYPE_BF16, DTYPE_F32, check, lib
 
 
 def _f32(a) -> np.ndarray:
@@ -97,6 +97,13 @@ class DecodeResidentState:
         """full_attention_bf16_for_test (attention.rs:47-54)."""
         return self.full_attention_with_element(capacity, q_heads, kv_heads, head_dim,
                                                 DTYPE_BF16, window)
+
+
+    def full_attention_f32(self, capacity, q_heads, kv_heads, head_dim, window=0):
+        """The f32 element of full_attention_with_element (attention.rs:56-108): what
+        full_attention chooses for greedy decoding."""
+        return self.full_attention_with_element(capacity, q_heads, kv_heads, head_dim,
+                                                DTYPE_F32, window)
 
 
 def rope_rotations(position, rope_dims, theta, position_scale=1.0, frequency_dim=0) -> np.ndarray:
@@ -214,9 +221,12 @@ class FullAttentionState:
         return k, v
 
     def read_rows_f32(self, first: int = 0, n: int | None = None):
-        k, v = self.read_rows(first, n)
-        return ((k.astype(np.uint32) << 16).view(np.float32),
-                (v.astype(np.uint32) << 16).view(np.float32))
+        """Logical rows as f32, for either element type (bf16 rows widen exactly)."""
+        n = self.len() - first if n is None else n
+        k = np.empty((n, self.kv_dim()), dtype=np.float32)
+        v = np.empty((n, self.kv_dim()), dtype=np.float32)
+        check(self._l.skv_read_rows_f32(self._h, first, n, _p(k), _p(v)))
+        return k, v
 
     # ---- device entry points (raw pointers + stream handle)
     def encode_append_kv(self, stream, k_ptr, v_ptr) -> None:

@@ -1,0 +1,199 @@
+"""The f32 element of the cache (KvElement::F32, src/decode_resident/attention.rs:26-108):
+what full_attention chooses for greedy decoding unless RETI_RUST_KV_BF16 says otherwise
+(src/decode_resident/utils.rs:202-229). Rows are kept verbatim, so contents are compared bit
+for bit with the oracle's f32 cache, and attention with cached_attention_one on it (the
+reference's own bound for its f32 GPU path is 1e-4, tests.rs:1443-1492; the bound to hold here
+is 1e-2)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+import saragossa_amd as skv
+from test_prekv_gpu import run_gated, run_prekv
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+TOL = 2e-5
+
+
+@pytest.fixture
+def env_flags():
+    saved = {k: os.environ.get(k) for k in ("RETI_RUST_KV_BF16",)}
+    yield os.environ
+    for k, v in saved.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
+    skv.flags.reload()
+
+
+def _filled(state, dims, n, seed, window=0, cap=None):
+    q_heads, kv_heads, head_dim = dims
+    kv_dim = kv_heads * head_dim
+    rng = np.random.default_rng(seed)
+    kv = state.full_attention_f32(cap or n + 8, q_heads, kv_heads, head_dim, window=window)
+    kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("f32")
+    keys = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    values = rng.standard_normal((n, kv_dim), dtype=np.float32)
+    if n:
+        kv.seed(keys, values, n)
+        cache.append_batch(keys, values, lay)
+    return kv, cache, lay, rng
+
+
+def test_policy_chooses_the_element(state, env_flags):
+    # kv_bf16_for: the override wins, else bf16 when sampling and f32 for greedy decoding
+    env_flags.pop("RETI_RUST_KV_BF16", None)
+    skv.flags.reload()
+    greedy = state.full_attention(64, 8, 2, 64, sampled=False)
+    sampled = state.full_attention(64, 8, 2, 64, sampled=True)
+    assert greedy.byte_len() == 64 * 2 * 64 * 4 and sampled.byte_len() == 64 * 2 * 64 * 2
+    env_flags["RETI_RUST_KV_BF16"] = "1"
+    skv.flags.reload()
+    assert state.full_attention(64, 8, 2, 64, sampled=False).byte_len() == 64 * 2 * 64 * 2
+    env_flags["RETI_RUST_KV_BF16"] = "off"
+    skv.flags.reload()
+    assert state.full_attention(64, 8, 2, 64, sampled=True).byte_len() == 64 * 2 * 64 * 4
+
+
+@pytest.mark.parametrize("dims", [(16, 2, 256), (32, 8, 128), (8, 8, 64), (6, 2, 96), (6, 1, 40), (4, 2, 16)])
+def test_rows_are_kept_verbatim(state, dims):
+    kv, cache, lay, rng = _filled(state, dims, 333, seed=dims[2])
+    kv_dim = dims[1] * dims[2]
+    special = np.array([0.0, -0.0, 1e-45, -1e-38, 3.4e38, np.inf, -np.inf, 1.0 + 2.0 ** -23], np.float32)
+    k1 = np.resize(special, kv_dim).astype(np.float32)
+    v1 = np.resize(special[::-1], kv_dim).astype(np.float32)
+    kv.append_row(k1, v1)
+    cache.append(k1[None], v1[None], lay)
+    gk, gv = kv.read_rows_f32()
+    assert np.array_equal(gk.view(np.uint32), cache.keys().view(np.uint32))
+    assert np.array_equal(gv.view(np.uint32), cache.values().view(np.uint32))
+    gk2, _ = kv.read_rows_f32(17, 40)
+    assert np.array_equal(gk2, cache.keys()[17:57])
+    with pytest.raises(skv.ConfigError):
+        kv.read_rows()  # bf16 bit patterns of an f32 layer
+    kv.truncate(100)
+    assert kv.len() == 100
+    with pytest.raises(skv.DimensionError):
+        kv.read_rows_f32(90, 20)
+
+
+@pytest.mark.parametrize("dims,n", [((16, 2, 256), 1), ((16, 2, 256), 257), ((16, 2, 256), 33000),
+                                    ((32, 8, 128), 4096), ((6, 1, 40), 1500), ((40, 1, 64), 700),
+                                    ((4, 4, 16), 100)])
+def test_attention_decode_matches_cpu(state, dims, n):
+    kv, cache, lay, rng = _filled(state, dims, n, seed=n)
+    q = rng.standard_normal(dims[0] * dims[2], dtype=np.float32)
+    got = kv.attention_decode(q)
+    want = oracle.cached_attention_one(q, cache, lay)
+    assert np.abs(got - want).max() <= TOL, np.abs(got - want).max()
+    # a window start inside the cache
+    if n > 20:
+        ws = n // 3
+        got = kv.attention_decode_windowed(q, ws)
+        sub = oracle.LayerKvCache("f32")
+        sub.append_batch(cache.keys()[ws:], cache.values()[ws:], lay)
+        assert np.abs(got - oracle.cached_attention_one(q, sub, lay)).max() <= TOL
+
+
+@pytest.mark.parametrize("dims,start,chunk", [((16, 2, 256), 5000, 300), ((32, 8, 128), 0, 700),
+                                               ((16, 2, 256), 5, 3), ((6, 1, 40), 100, 100)])
+def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk):
+    q_heads, kv_heads, head_dim = dims
+    kv, cache, lay, rng = _filled(state, dims, start, seed=start + chunk, cap=start + chunk)
+    q = rng.standard_normal((chunk, q_heads * head_dim), dtype=np.float32)
+    k = rng.standard_normal((chunk, kv_heads * head_dim), dtype=np.float32)
+    v = rng.standard_normal((chunk, kv_heads * head_dim), dtype=np.float32)
+    got = kv.prefill_rows(q, k, v)
+    want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+    assert np.abs(got - want).max() <= TOL, np.abs(got - want).max()
+    gk, gv = kv.read_rows_f32()
+    assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
+
+
+def test_ring_layer_chunks_and_steps(state):
+    dims, window = (8, 2, 64), 100
+    kv, cache, lay, rng = _filled(state, dims, 0, seed=5, window=window, cap=2000)
+    q_dim, kv_dim = dims[0] * dims[2], dims[1] * dims[2]
+    for chunk in (70, 1, 250, 33, 1, 1, 112):
+        q = rng.standard_normal((chunk, q_dim), dtype=np.float32)
+        k = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+        v = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+        got = kv.prefill_rows(q, k, v)
+        want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+        assert np.abs(got - want).max() <= TOL
+    n = kv.len()
+    gk, gv = kv.read_rows_f32(n - window, window)
+    assert np.array_equal(gk, cache.keys()[n - window:]) and np.array_equal(gv, cache.values()[n - window:])
+
+
+def test_snapshot_restore_and_hot_cache_on_f32_layers(state):
+    dims = (8, 2, 128)
+    layers, caches = [], []
+    for li in range(3):
+        kv, cache, lay, rng = _filled(state, dims, 160, seed=40 + li, cap=400)
+        layers.append(kv)
+        caches.append(cache)
+    snap = skv.snapshot_blocks(state, layers, [1, 4, 9])
+    assert snap.estimated_bytes() == 3 * 3 * 2 * 16 * dims[1] * dims[2] * 4
+    others = [_filled(state, dims, 160, seed=90 + li, cap=400)[0] for li in range(3)]
+    skv.restore_blocks(state, snap, others, [1, 4, 9])
+    for kv, cache in zip(others, caches):
+        gk, gv = kv.read_rows_f32()
+        for p in (1, 4, 9):
+            assert np.array_equal(gk[p * 16:(p + 1) * 16], cache.keys()[p * 16:(p + 1) * 16])
+            assert np.array_equal(gv[p * 16:(p + 1) * 16], cache.values()[p * 16:(p + 1) * 16])
+    # the hot cache: remember two blocks of 32 tokens, restore them into fresh layers
+    hot = skv.HotCache(state, 32, 8, 8, layers)
+    root = skv.BlockHash.root()
+    tokens = list(range(64))
+    h1 = skv.BlockHash.chain(root, tokens[:32])
+    h2 = skv.BlockHash.chain(h1, tokens[32:])
+    assert hot.remember_prefix_block(root, h1, 32, layers)
+    assert hot.remember_prefix_block(root, h2, 64, layers)
+    fresh = [state.full_attention_f32(400, *dims) for _ in range(3)]
+    assert hot.match_restore(root, tokens + [7, 8, 9], fresh)[0] == 64
+    for kv, cache in zip(fresh, caches):
+        assert kv.len() == 64
+        gk, gv = kv.read_rows_f32()
+        assert np.array_equal(gk, cache.keys()[:64]) and np.array_equal(gv, cache.values()[:64])
+    # layers of the other element do not fit the pool
+    with pytest.raises(skv.KvError):
+        hot.remember_prefix_block(root, h1, 32, [state.full_attention_bf16(400, *dims) for _ in range(3)])
+
+
+def test_device_steps_on_f32_layers(state):
+    # the fused entry points run as separate launches on an f32 layer
+    run_prekv(state, (16, 2, 256), 0, 300, 6, 64, 1.0e7, None, (True, True), element="f32")
+    run_prekv(state, (8, 2, 64), 40, 100, 30, 64, 1.0e6, None, (True, False), element="f32")
+    run_gated(state, (16, 2, 256), 0, 200, 5, 64, 1.0e7, element="f32")
+
+
+def test_decode_step_batch_on_f32_layers(state):
+    dims = (16, 2, 256)
+    q_dim, kv_dim = dims[0] * dims[2], dims[1] * dims[2]
+    seqs = [_filled(state, dims, n, seed=n) for n in (50, 700, 3000)]
+    rng = np.random.default_rng(3)
+    for _ in range(3):
+        rows = [(rng.standard_normal(kv_dim, dtype=np.float32), rng.standard_normal(kv_dim, dtype=np.float32),
+                 rng.standard_normal(q_dim, dtype=np.float32)) for _ in seqs]
+        dev = [[torch.from_numpy(a).cuda() for a in r] for r in rows]
+        outs = [torch.empty(q_dim, device="cuda") for _ in seqs]
+        skv.encode_decode_step_batch([s[0] for s in seqs], torch.cuda.current_stream().cuda_stream,
+                                     [d[0].data_ptr() for d in dev], [d[1].data_ptr() for d in dev],
+                                     [d[2].data_ptr() for d in dev], [o.data_ptr() for o in outs])
+        for (kv, cache, lay, _), (k, v, q), o in zip(seqs, rows, outs):
+            want = oracle.decode_step(cache, k, v, q, lay)
+            assert np.abs(o.cpu().numpy() - want).max() <= TOL
+
+
+def test_head_dim_above_256_is_rejected_loudly(state):
+    with pytest.raises(skv.ConfigError):
+        state.full_attention_f32(64, 4, 1, 320)

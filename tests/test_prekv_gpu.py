@@ -138,16 +138,17 @@ CASES = [
 ]
 
 
-def run_prekv(state, dims, window, start, steps, rope_dims, theta, attn_scalar, norms):
+def run_prekv(state, dims, window, start, steps, rope_dims, theta, attn_scalar, norms, element="bf16"):
     q_heads, kv_heads, head_dim = dims
     kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
     eps = 1.0e-6
     rng = np.random.default_rng(start * 7 + steps)
     cap = start + steps
-    kv = state.full_attention_bf16(cap, q_heads, kv_heads, head_dim, window=window)
+    make = state.full_attention_f32 if element == "f32" else state.full_attention_bf16
+    kv = make(cap, q_heads, kv_heads, head_dim, window=window)
     kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
     lay = oracle.layout(q_heads, kv_heads, head_dim, attn_scalar=attn_scalar, sliding_window=window)
-    cache = oracle.LayerKvCache("bf16r")
+    cache = oracle.LayerKvCache("f32" if element == "f32" else "bf16r")
     q_norm = (0.7 + np.abs(pseudo(np.arange(head_dim) * 11))).astype(np.float32)
     k_norm = (0.8 + np.abs(pseudo(np.arange(head_dim) * 17))).astype(np.float32)
 
@@ -275,16 +276,17 @@ GATED = [
 ]
 
 
-def run_gated(state, dims, window, start, steps, rope_dims, theta):
+def run_gated(state, dims, window, start, steps, rope_dims, theta, element="bf16"):
     q_heads, kv_heads, head_dim = dims
     kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
     eps = 1.0e-6
     rng = np.random.default_rng(start * 5 + steps)
     cap = start + steps
-    kv = state.full_attention_bf16(cap, q_heads, kv_heads, head_dim, window=window)
+    make = state.full_attention_f32 if element == "f32" else state.full_attention_bf16
+    kv = make(cap, q_heads, kv_heads, head_dim, window=window)
     kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
     lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
-    cache = oracle.LayerKvCache("bf16r")
+    cache = oracle.LayerKvCache("f32" if element == "f32" else "bf16r")
     q_norm = (0.7 + np.abs(pseudo(np.arange(head_dim) * 11))).astype(np.float32)
     k_norm = (0.8 + np.abs(pseudo(np.arange(head_dim) * 17))).astype(np.float32)
     if start:
