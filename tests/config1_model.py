@@ -57,12 +57,14 @@ def norm_rope(x, heads, head_dim, w, eps, theta, positions):
 
 class HipKv:
     """KV path on the HIP library: paged bf16 caches behind permuted block tables."""
+    ELEMENT = "bf16"
 
     def __init__(self, cfg, capacity, state, seed=0):
         rng = np.random.default_rng(seed)
         self.layers = []
+        make = state.full_attention_f32 if self.ELEMENT == "f32" else state.full_attention_bf16
         for _ in range(cfg.layers):
-            kv = state.full_attention_bf16(capacity, cfg.q_heads, cfg.kv_heads, cfg.head_dim)
+            kv = make(capacity, cfg.q_heads, cfg.kv_heads, cfg.head_dim)
             kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
             self.layers.append(kv)
         self.stream = torch.cuda.current_stream().cuda_stream
@@ -84,10 +86,11 @@ class HipKv:
 
 class OracleKv:
     """KV path on the CPU oracle with K/V rounded to bf16 at append (mode bf16r)."""
+    MODE = "bf16r"
 
     def __init__(self, cfg, capacity=None, state=None, seed=0):
         self.lay = oracle.layout(cfg.q_heads, cfg.kv_heads, cfg.head_dim)
-        self.caches = [oracle.LayerKvCache("bf16r") for _ in range(cfg.layers)]
+        self.caches = [oracle.LayerKvCache(self.MODE) for _ in range(cfg.layers)]
 
     def attend(self, li, q, k, v):
         qn, kn, vn = q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
@@ -99,6 +102,16 @@ class OracleKv:
 
     def contents(self, li):
         return self.caches[li].keys(), self.caches[li].values()
+
+
+class HipKvF32(HipKv):
+    """The same with the f32 element: the reference's choice for greedy decoding."""
+    ELEMENT = "f32"
+
+
+class OracleKvF32(OracleKv):
+    """The CPU path as it is: f32 rows."""
+    MODE = "f32"
 
 
 def norm_rope_cpu(x, heads, cfg, position):

@@ -12,17 +12,19 @@ import pytest
 pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
-from config1_model import Config, HipKv, HipKvPre, OracleKv, OracleKvPre, Weights, greedy  # noqa: E402
+from config1_model import (Config, HipKv, HipKvF32, HipKvPre, OracleKv, OracleKvF32, OracleKvPre,  # noqa: E402
+                           Weights, greedy)
 
 FULL = os.environ.get("SKV_FULL_CONFIG1") == "1"
 
 
 @pytest.mark.timeout(3000 if FULL else 300)
-@pytest.mark.parametrize("hip_cls,ora_cls", [(HipKv, OracleKv), (HipKvPre, OracleKvPre)],
-                         ids=["kv-path", "fused-pre-kv"])
+@pytest.mark.parametrize("hip_cls,ora_cls", [(HipKv, OracleKv), (HipKvPre, OracleKvPre), (HipKvF32, OracleKvF32)],
+                         ids=["kv-path", "fused-pre-kv", "f32-element"])
 def test_config1_greedy_ids_match_oracle(state, hip_cls, ora_cls):
     """ids "fused-pre-kv": decode tokens additionally run the q/k norms and the rotation
-    inside the library's fused step (device) against rms_norm_rope_heads_at (CPU)."""
+    inside the library's fused step (device) against rms_norm_rope_heads_at (CPU).
+    "f32-element": both arms keep f32 rows, as the reference does for greedy decoding."""
     cfg = Config() if FULL else Config(layers=4)
     n_prompt, n_new, chunk = (2048, 256, 512) if FULL else (256, 48, 96)
     w = Weights(cfg, seed=1)
