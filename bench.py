@@ -158,19 +158,21 @@ def bench_restore(skv, torch, np, state, stream):
     return out
 
 
-def bench_prefill(skv, torch, np, state, stream):
+def bench_prefill(skv, torch, np, state, stream, element="bf16"):
     """Chunked prefill over the cache (cached_attention_prefill_rows as one launch): a
     512-row chunk appended and attended causally over the rows already cached, at the KV
     shapes of configs[2] (after 32768 rows) and configs[1] (the last chunk of its 2048-token
     prompt). The one matrix-core-bound kernel of the path: flops = 4 * keys * q_dim over the
     (query, key) pairs attended; the kernel issues twice that on the matrix cores because
-    queries and probabilities are split into two bf16 terms."""
+    queries and probabilities are split into two bf16 terms. With the f32 element the products
+    run once, on the f32 matrix instruction."""
     dev = torch.device("cuda:0")
+    f32 = element == "f32"
     out = []
     for name, (qh, kvh, hd), base, chunk in (("configs[2] shape q16/kv2/hd256", (16, 2, 256), 32768, 512),
                                             ("configs[1] shape q32/kv8/hd128", (32, 8, 128), 1536, 512)):
         kv_dim, q_dim = kvh * hd, qh * hd
-        kv = state.full_attention_bf16(base + chunk + 16, qh, kvh, hd)
+        kv = (state.full_attention_f32 if f32 else state.full_attention_bf16)(base + chunk + 16, qh, kvh, hd)
         kv.set_block_table(np.random.default_rng(7).permutation(kv.pages()).astype(np.int32))
         gen = torch.Generator(device=dev)
         gen.manual_seed(7)
@@ -196,11 +198,15 @@ def bench_prefill(skv, torch, np, state, stream):
         us = ts[len(ts) // 2]
         keys = sum(base + i + 1 for i in range(chunk))
         flops = 4 * keys * q_dim
-        out.append({"workload": "%s: %d-row chunk over %d cached rows (append + attention + merge)"
-                                % (name, chunk, base),
-                    "us": round(us, 1), "algorithmic_tflops": round(flops / us / 1e6, 1),
-                    "mfma_tflops_issued": round(2 * flops / us / 1e6, 1),
-                    "frac_of_bf16_mfma_peak": round(2 * flops / us / 1e6 / 2500.0, 4)})
+        row = {"workload": "%s, %s element: %d-row chunk over %d cached rows (append + attention + merge)"
+                           % (name, element, chunk, base),
+               "us": round(us, 1), "algorithmic_tflops": round(flops / us / 1e6, 1)}
+        if f32:
+            row["frac_of_f32_mfma_peak"] = round(flops / us / 1e6 / 157.3, 4)
+        else:
+            row["mfma_tflops_issued"] = round(2 * flops / us / 1e6, 1)
+            row["frac_of_bf16_mfma_peak"] = round(2 * flops / us / 1e6 / 2500.0, 4)
+        out.append(row)
         kv.close()
     return out
 
@@ -731,7 +737,7 @@ def main() -> int:
     if args.config == 1 and args.end_to_end:
         result["end_to_end"] = bench_end_to_end(skv, torch, np, state)
     if args.config == 2 and not args.no_restore:
-        result["prefill"] = bench_prefill(skv, torch, np, state, stream)
+        result["prefill"] = bench_prefill(skv, torch, np, state, stream, args.element)
 
     if not args.no_cpu_baseline:
         import oracle
