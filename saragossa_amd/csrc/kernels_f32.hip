@@ -148,6 +148,25 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     const int pb0 = page_lo + (int)(((unsigned)split * span) / (unsigned)a.splits);
     const int pb1 = page_lo + (int)(((unsigned)(split + 1) * span) / (unsigned)a.splits);
 
+    const float *k_pool = reinterpret_cast<const float *>(a.k_pool);
+    const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
+    const int last_page = a.page_first + a.n_pages - 1;
+    // (every page of [page_lo, page_hi) is visible to some slot of the tile)
+    auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
+        const int page = a.table[min(pb, last_page)];
+        const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
+        const float4_t *kt = reinterpret_cast<const float4_t *>(k_pool + tile);
+        const float4_t *vt = reinterpret_cast<const float4_t *>(v_pool + tile);
+#pragma unroll
+        for (int m = 0; m < NT; ++m) kq[m] = kt[m * 64 + lane];
+#pragma unroll
+        for (int c = 0; c < NT; ++c) vq[c] = vt[c * 64 + lane];
+    };
+    // The first page is requested before anything else: the queries' loads ride behind it.
+    float4_t k_a[NT], v_a[NT], k_b[NT], v_b[NT];
+    int pb = pb0 + wave;
+    if (pb < pb1) fetch(pb, k_a, v_a);
+
     // queries: lane (slot n, group j) holds dims 16m + 4j .. +3 of every block m
     float4_t qv[NT];
     {
@@ -176,20 +195,6 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     for (int c = 0; c < NT; ++c) o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
 
-    const float *k_pool = reinterpret_cast<const float *>(a.k_pool);
-    const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
-    const int last_page = a.page_first + a.n_pages - 1;
-    // (every page of [page_lo, page_hi) is visible to some slot of the tile)
-    auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
-        const int page = a.table[min(pb, last_page)];
-        const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
-        const float4_t *kt = reinterpret_cast<const float4_t *>(k_pool + tile);
-        const float4_t *vt = reinterpret_cast<const float4_t *>(v_pool + tile);
-#pragma unroll
-        for (int m = 0; m < NT; ++m) kq[m] = kt[m * 64 + lane];
-#pragma unroll
-        for (int c = 0; c < NT; ++c) vq[c] = vt[c * 64 + lane];
-    };
     auto consume = [&](int pb, const float4_t (&kq)[NT], const float4_t (&vq)[NT]) {
         const int slot_a = pb * 16; // first cache slot of the page
         // S^T = K . Q^T: two accumulators so that consecutive products do not wait for each other
@@ -242,9 +247,6 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     // The page after the one being multiplied is already on its way into a second set of
     // registers: without that every wavefront of the device loads, then multiplies, in step,
     // and memory idles half the time.
-    float4_t k_a[NT], v_a[NT], k_b[NT], v_b[NT];
-    int pb = pb0 + wave;
-    if (pb < pb1) fetch(pb, k_a, v_a);
     while (pb < pb1) {
         if (pb + 4 < pb1) fetch(pb + 4, k_b, v_b);
         consume(pb, k_a, v_a);
