@@ -14,8 +14,9 @@
  *
  * Layout: the cache of one layer is a pool of 16-token pages reached through a
  * block table; logical row r of the reference's contiguous cache is
- * (block_table[r / 16], r % 16) here. Elements are bf16, rounded from f32 with
- * the reference's integer formula (src/decode_resident/utils.rs:55-60).
+ * (block_table[r / 16], r % 16) here. A layer's elements are bf16, rounded from
+ * f32 with the reference's integer formula (src/decode_resident/utils.rs:55-60),
+ * or f32 kept verbatim (GpuElement, src/decode_resident/attention.rs:26-45).
  */
 #ifndef SARAGOSSA_KV_H
 #define SARAGOSSA_KV_H
