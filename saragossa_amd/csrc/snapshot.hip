@@ -156,15 +156,23 @@ static int32_t launch_flat(const void *const *src, void *const *dst, const size_
 // Shapes of the layers a storage area was laid out for.
 struct SlotLayout {
     std::vector<uint32_t> page_bytes; // per layer
+    std::vector<uint64_t> shape;      // per layer: what the bytes of a page mean
     std::vector<uint64_t> slot_off;
     uint64_t slot_bytes = 0;
 
+    // kv heads, head_dim and element: two layers whose pages merely have the same size
+    // (bf16 at head_dim 256 and f32 at 128, say) must not exchange pages
+    static uint64_t shape_of(const skv_layer *L) {
+        return ((uint64_t)L->g.kv_heads << 32) | ((uint64_t)L->g.head_dim << 1) | (uint64_t)(L->g.f32 & 1);
+    }
     void build(skv_layer *const *layers, size_t n) {
         page_bytes.resize(n);
+        shape.resize(n);
         slot_off.resize(n);
         slot_bytes = 0;
         for (size_t i = 0; i < n; ++i) {
             page_bytes[i] = (uint32_t)((size_t)layers[i]->g.page_elems * sizeof(uint16_t));
+            shape[i] = shape_of(layers[i]);
             slot_off[i] = slot_bytes;
             slot_bytes += 2ull * page_bytes[i];
         }
@@ -172,7 +180,7 @@ struct SlotLayout {
     bool matches(skv_layer *const *layers, size_t n) const {
         if (n != page_bytes.size()) return false;
         for (size_t i = 0; i < n; ++i)
-            if (page_bytes[i] != (uint32_t)((size_t)layers[i]->g.page_elems * sizeof(uint16_t))) return false;
+            if (shape[i] != shape_of(layers[i])) return false;
         return true;
     }
 };

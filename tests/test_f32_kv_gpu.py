@@ -164,9 +164,14 @@ def test_snapshot_restore_and_hot_cache_on_f32_layers(state):
         assert kv.len() == 64
         gk, gv = kv.read_rows_f32()
         assert np.array_equal(gk, cache.keys()[:64]) and np.array_equal(gv, cache.values()[:64])
-    # layers of the other element do not fit the pool
+    # layers of the other element do not fit the pool, not even when their pages have the
+    # same size (bf16 at twice the head_dim)
     with pytest.raises(skv.KvError):
         hot.remember_prefix_block(root, h1, 32, [state.full_attention_bf16(400, *dims) for _ in range(3)])
+    with pytest.raises(skv.KvError):
+        hot.remember_prefix_block(root, h1, 32, [state.full_attention_bf16(400, 8, 2, 256) for _ in range(3)])
+    with pytest.raises(skv.KvError):
+        skv.restore_blocks(state, snap, [state.full_attention_bf16(400, 8, 2, 256) for _ in range(3)], [1, 4, 9])
 
 
 def test_device_steps_on_f32_layers(state):
