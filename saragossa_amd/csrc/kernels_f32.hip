@@ -152,20 +152,28 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
     const int last_page = a.page_first + a.n_pages - 1;
     // (every page of [page_lo, page_hi) is visible to some slot of the tile)
-    auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
+    auto fetch_tile = [&](int pb, const float *pool, float4_t (&dst)[NT]) {
         const int page = a.table[min(pb, last_page)];
         const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
-        const float4_t *kt = reinterpret_cast<const float4_t *>(k_pool + tile);
-        const float4_t *vt = reinterpret_cast<const float4_t *>(v_pool + tile);
+        const float4_t *t = reinterpret_cast<const float4_t *>(pool + tile);
 #pragma unroll
-        for (int m = 0; m < NT; ++m) kq[m] = kt[m * 64 + lane];
-#pragma unroll
-        for (int c = 0; c < NT; ++c) vq[c] = vt[c * 64 + lane];
+        for (int m = 0; m < NT; ++m) dst[m] = t[m * 64 + lane];
     };
-    // The first page is requested before anything else: the queries' loads ride behind it.
-    float4_t k_a[NT], v_a[NT], k_b[NT], v_b[NT];
+    auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
+        fetch_tile(pb, k_pool, kq);
+        fetch_tile(pb, v_pool, vq);
+    };
+    // Up to head_dim 256 a wavefront holds two pages (K and V each); above, one tile at a
+    // time (K, then V in the same registers). The first page is requested before anything
+    // else: the queries' loads ride behind it.
+    constexpr bool TWO_PAGES = P <= 256;
+    constexpr int NB = TWO_PAGES ? NT : 1;
+    float4_t k_a[NT], v_a[NB], k_b[NB], v_b[NB];
     int pb = pb0 + wave;
-    if (pb < pb1) fetch(pb, k_a, v_a);
+    if (pb < pb1) {
+        if constexpr (TWO_PAGES) fetch(pb, k_a, v_a);
+        else fetch_tile(pb, k_pool, k_a);
+    }
 
     // queries: lane (slot n, group j) holds dims 16m + 4j .. +3 of every block m
     float4_t qv[NT];
@@ -195,7 +203,8 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     for (int c = 0; c < NT; ++c) o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
 
-    auto consume = [&](int pb, const float4_t (&kq)[NT], const float4_t (&vq)[NT]) {
+    // scores and probabilities of one page (pv), running state updated
+    auto attend = [&](int pb, const float4_t (&kq)[NT], float (&pv)[4]) {
         const int slot_a = pb * 16; // first cache slot of the page
         // S^T = K . Q^T: two accumulators so that consecutive products do not wait for each other
         float4_t s0 = float4_t{0.f, 0.f, 0.f, 0.f}, s1 = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -224,7 +233,6 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
         const float m_new = fmaxf(m_run, m_blk);
         const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = fast_exp2(m_run - m_safe);
-        float pv[4];
         float psum = 0.0f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -237,24 +245,43 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
 #pragma unroll
             for (int c = 0; c < NT; ++c) o[c] *= alpha;
         }
-        // O^T += V^T . P^T, contraction step outermost: consecutive products use different accumulators
+    };
+    // O^T += V^T . P^T, contraction step outermost: consecutive products use different accumulators
+    auto accumulate = [&](const float4_t (&vq)[NT], const float (&pv)[4]) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
 #pragma unroll
             for (int c = 0; c < NT; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq[c][k], pv[k], o[c], 0, 0, 0);
         }
     };
-    // The page after the one being multiplied is already on its way into a second set of
-    // registers: without that every wavefront of the device loads, then multiplies, in step,
-    // and memory idles half the time.
-    while (pb < pb1) {
-        if (pb + 4 < pb1) fetch(pb + 4, k_b, v_b);
-        consume(pb, k_a, v_a);
-        pb += 4;
-        if (pb >= pb1) break;
-        if (pb + 4 < pb1) fetch(pb + 4, k_a, v_a);
-        consume(pb, k_b, v_b);
-        pb += 4;
+    if constexpr (TWO_PAGES) {
+        // The page after the one being multiplied is already on its way into a second set of
+        // registers: without that every wavefront of the device loads, then multiplies, in
+        // step, and memory idles half the time.
+        auto consume = [&](int at, const float4_t (&kq)[NT], const float4_t (&vq)[NT]) {
+            float pv[4];
+            attend(at, kq, pv);
+            accumulate(vq, pv);
+        };
+        while (pb < pb1) {
+            if (pb + 4 < pb1) fetch(pb + 4, k_b, v_b);
+            consume(pb, k_a, v_a);
+            pb += 4;
+            if (pb >= pb1) break;
+            if (pb + 4 < pb1) fetch(pb + 4, k_a, v_a);
+            consume(pb, k_b, v_b);
+            pb += 4;
+        }
+    } else {
+        // head_dim 257..512: the queries and the accumulators are 256 registers by themselves;
+        // K, then V of the page, then K of the next one pass through the same 128
+        for (; pb < pb1; pb += 4) {
+            float pv[4];
+            attend(pb, k_a, pv);
+            fetch_tile(pb, v_pool, k_a);
+            accumulate(k_a, pv);
+            if (pb + 4 < pb1) fetch_tile(pb + 4, k_pool, k_a);
+        }
     }
 
     // ---- the four wavefronts' states meet in LDS ------------------------------------------
@@ -335,6 +362,7 @@ hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
     case 64: return launch_f32<64>(a, grid, s);
     case 128: return launch_f32<128>(a, grid, s);
     case 256: return launch_f32<256>(a, grid, s);
+    case 512: return launch_f32<512>(a, grid, s);
     default: return hipErrorInvalidValue;
     }
 }

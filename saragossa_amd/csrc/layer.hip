@@ -500,7 +500,6 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     const bool f32 = dtype == SKV_DTYPE_F32;
     const int P = padded_head_dim(head_dim);
     if (P == 0) return fail(SKV_ERR_CONFIG, "head_dim > 512 non supporté");
-    if (f32 && P > 256) return fail(SKV_ERR_CONFIG, "KV f32: head_dim > 256 non supporté");
     if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096)
         return fail(SKV_ERR_CONFIG, "capacité KV déborde");
     SKV_HIP(hipSetDevice(ctx->device));

@@ -63,7 +63,8 @@ def test_policy_chooses_the_element(state, env_flags):
     assert state.full_attention(64, 8, 2, 64, sampled=True).byte_len() == 64 * 2 * 64 * 4
 
 
-@pytest.mark.parametrize("dims", [(16, 2, 256), (32, 8, 128), (8, 8, 64), (6, 2, 96), (6, 1, 40), (4, 2, 16)])
+@pytest.mark.parametrize("dims", [(16, 2, 256), (32, 8, 128), (8, 8, 64), (6, 2, 96), (6, 1, 40), (4, 2, 16),
+                                  (4, 1, 320), (8, 2, 512)])
 def test_rows_are_kept_verbatim(state, dims):
     kv, cache, lay, rng = _filled(state, dims, 333, seed=dims[2])
     kv_dim = dims[1] * dims[2]
@@ -87,7 +88,7 @@ def test_rows_are_kept_verbatim(state, dims):
 
 @pytest.mark.parametrize("dims,n", [((16, 2, 256), 1), ((16, 2, 256), 257), ((16, 2, 256), 33000),
                                     ((32, 8, 128), 4096), ((6, 1, 40), 1500), ((40, 1, 64), 700),
-                                    ((4, 4, 16), 100)])
+                                    ((4, 4, 16), 100), ((8, 2, 512), 9000), ((4, 1, 320), 300)])
 def test_attention_decode_matches_cpu(state, dims, n):
     kv, cache, lay, rng = _filled(state, dims, n, seed=n)
     q = rng.standard_normal(dims[0] * dims[2], dtype=np.float32)
@@ -104,7 +105,8 @@ def test_attention_decode_matches_cpu(state, dims, n):
 
 
 @pytest.mark.parametrize("dims,start,chunk", [((16, 2, 256), 5000, 300), ((32, 8, 128), 0, 700),
-                                               ((16, 2, 256), 5, 3), ((6, 1, 40), 100, 100)])
+                                               ((16, 2, 256), 5, 3), ((6, 1, 40), 100, 100),
+                                               ((4, 1, 512), 700, 150)])
 def test_prefill_rows_match_per_row_oracle(state, dims, start, chunk):
     q_heads, kv_heads, head_dim = dims
     kv, cache, lay, rng = _filled(state, dims, start, seed=start + chunk, cap=start + chunk)
@@ -199,6 +201,6 @@ def test_decode_step_batch_on_f32_layers(state):
             assert np.abs(o.cpu().numpy() - want).max() <= TOL
 
 
-def test_head_dim_above_256_is_rejected_loudly(state):
+def test_head_dim_above_512_is_rejected_loudly(state):
     with pytest.raises(skv.ConfigError):
-        state.full_attention_f32(64, 4, 1, 320)
+        state.full_attention_f32(64, 4, 1, 520)

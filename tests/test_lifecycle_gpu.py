@@ -41,8 +41,6 @@ def _check_contents(kv, cache, window):
 def test_random_lifetime_matches_the_oracle(state, seed, element):
     rng = np.random.default_rng(1000 + seed)
     q_heads, kv_heads, head_dim = GEOMETRIES[seed % len(GEOMETRIES)]
-    if element == "f32" and head_dim > 256:
-        pytest.skip("the f32 element is built up to head_dim 256")
     make = state.full_attention_f32 if element == "f32" else state.full_attention_bf16
     kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
     window = 0 if seed % 3 else int(rng.integers(17, 90))
