@@ -120,7 +120,8 @@ int32_t skv_ctx_synchronize(skv_ctx *ctx);
  * (rounded up to whole pages); 0 keeps all `capacity` rows in pages.
  * `dtype` is what the pages hold: SKV_DTYPE_BF16 (rows rounded to nearest even at append,
  * pages of kv_heads * P * 32 bytes per tensor, P = head_dim rounded up to a power of two) or
- * SKV_DTYPE_F32 (rows verbatim; pages twice the bytes). head_dim up to 512 in both. Every entry point below serves both; where they differ it says so. */
+ * SKV_DTYPE_F32 (rows verbatim; pages twice the bytes). head_dim up to 512 in both. Every
+ * entry point below serves both; where they differ it says so. */
 int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
                          size_t head_dim, int32_t dtype, size_t window, skv_layer **out);
 /* full_attention(capacity, q_heads, kv_heads, head_dim, sampled) (attention.rs:26-45):
