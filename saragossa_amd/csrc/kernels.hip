@@ -245,9 +245,10 @@ __global__ __launch_bounds__(256) void naive_kernel(NaiveArgs a) {
         const int page = a.table[slot >> 4];
         const int r = (int)(slot & 15);
         const uint16_t *kt = a.k_pool + (long)page * g.page_elems + (long)kvh * g.tile_elems;
+        const float *ktf = reinterpret_cast<const float *>(kt);
         float dot = 0.0f;
         for (int d = 0; d < g.head_dim; ++d)
-            dot = __fadd_rn(dot, __fmul_rn(q[d], bf16_to_f32(kt[k_index(g.P, r, d)])));
+            dot = __fadd_rn(dot, __fmul_rn(q[d], g.f32 ? ktf[k_index_f32(r, d)] : bf16_to_f32(kt[k_index(g.P, r, d)])));
         const float sc = __fmul_rn(dot, a.inv_scale);
         scores[i] = sc;
         mx = fmaxf(mx, sc);
@@ -282,7 +283,8 @@ __global__ __launch_bounds__(256) void naive_kernel(NaiveArgs a) {
             const int r = (int)(slot & 15);
             const uint16_t *vt = a.v_pool + (long)page * g.page_elems + (long)kvh * g.tile_elems;
             const float pr = uniform ? 1.0f / (float)nkeys : scores[i] / sum;
-            acc = __fadd_rn(acc, __fmul_rn(pr, bf16_to_f32(vt[v_index(g.P, r, d)])));
+            const float val = g.f32 ? reinterpret_cast<const float *>(vt)[v_index_f32(r, d)] : bf16_to_f32(vt[v_index(g.P, r, d)]);
+            acc = __fadd_rn(acc, __fmul_rn(pr, val));
         }
         a.out[(long)h * g.head_dim + d] = acc;
     }

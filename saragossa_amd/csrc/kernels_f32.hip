@@ -16,13 +16,6 @@ namespace skv {
 
 typedef __attribute__((ext_vector_type(4))) float float4_t;
 
-__host__ __device__ inline int k_index_f32(int r, int d) {
-    return (((d >> 4) * 64 + ((d >> 2) & 3) * 16 + r) << 2) + (d & 3);
-}
-__host__ __device__ inline int v_index_f32(int r, int d) {
-    return (((d >> 4) * 64 + (r >> 2) * 16 + (d & 15)) << 2) + (r & 3);
-}
-
 namespace {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 } // namespace

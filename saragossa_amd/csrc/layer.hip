@@ -286,10 +286,9 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     int32_t rc = check_window(L, window_start);
     if (rc) return rc;
     const Geom &g = L->g;
-    if (g.f32) {
-        // the f32 storage mode has one attention kernel (no plain variant, no fused append or
-        // pre-KV step): 16 query slots per workgroup, the context split while that leaves
-        // compute units idle
+    if (g.f32 && (uses_flash(L) || n_queries > 1)) {
+        // the f32 element's matrix kernel (no fused append or pre-KV step): 16 query slots per
+        // workgroup, the context split while that leaves compute units idle
         if (k_new || v_new || pre) return fail(SKV_ERR_CONFIG, "KV f32: étape fusionnée non construite");
         DecodeArgs a{};
         fill_decode_args(L, q_dev, out_dev, window_start, nullptr, nullptr, n_queries, decode_target_wgs(), a);

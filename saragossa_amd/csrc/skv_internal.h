@@ -73,6 +73,14 @@ __host__ __device__ inline int v_index(int P, int r, int d) {
     return ((((((d >> 5) * 4 + (r >> 2)) * 16 + (d & 15)) * 2 + ((d >> 4) & 1))) << 2) + (r & 3);
 }
 
+// The f32 element's tiles (kernels_f32.hip), in floats from the tile's start.
+__host__ __device__ inline int k_index_f32(int r, int d) {
+    return (((d >> 4) * 64 + ((d >> 2) & 3) * 16 + r) << 2) + (d & 3);
+}
+__host__ __device__ inline int v_index_f32(int r, int d) {
+    return (((d >> 4) * 64 + (r >> 2) * 16 + (d & 15)) << 2) + (r & 3);
+}
+
 // Rows are addressed by position; a ring layer keeps position p in slot p % ring_rows.
 __host__ __device__ inline long slot_of(long pos, int ring_rows) {
     return ring_rows > 0 ? pos % ring_rows : pos;

@@ -204,3 +204,28 @@ def test_decode_step_batch_on_f32_layers(state):
 def test_head_dim_above_512_is_rejected_loudly(state):
     with pytest.raises(skv.ConfigError):
         state.full_attention_f32(64, 4, 1, 520)
+
+
+@pytest.mark.parametrize("dims,n", [((16, 2, 256), 700), ((6, 1, 40), 300), ((4, 1, 320), 90)])
+def test_flash_sdpa_off_uses_the_plain_kernel_on_f32_rows(state, dims, n):
+    """RETI_RUST_FLASH_SDPA=0 (src/decode_resident/utils.rs:182-185): the plain three-phase
+    kernel reads the f32 tiles too; its sequential sums are an independent check of the matrix
+    kernel."""
+    kv, cache, lay, rng = _filled(state, dims, n, seed=n)
+    q = rng.standard_normal(dims[0] * dims[2], dtype=np.float32)
+    want = oracle.cached_attention_one(q, cache, lay)
+    saved = os.environ.get("RETI_RUST_FLASH_SDPA")
+    try:
+        os.environ["RETI_RUST_FLASH_SDPA"] = "0"
+        skv.flags.reload()
+        assert not skv.flags.flash_sdpa_enabled()
+        plain = kv.attention_decode(q)
+    finally:
+        if saved is None:
+            os.environ.pop("RETI_RUST_FLASH_SDPA", None)
+        else:
+            os.environ["RETI_RUST_FLASH_SDPA"] = saved
+        skv.flags.reload()
+    matrix = kv.attention_decode(q)
+    assert np.abs(plain - want).max() <= 2e-6
+    assert np.abs(plain - matrix).max() <= TOL
