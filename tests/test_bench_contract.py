@@ -1,0 +1,53 @@
+"""bench.py's command line and its one-line JSON, as far as they can be checked without a GPU:
+more than one GPU is refused with a message, the byte count behind `roofline.achieved` is the
+stated formula, and (on the GPU) the default run prints one JSON object with the agreed keys."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "bench.py")
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert r.stdout.strip() == ""
+    assert "one GPU" in r.stderr
+
+
+def test_algorithmic_bytes_formula():
+    sys.path.insert(0, ROOT)
+    import bench
+    rows, kv_dim, q_dim = 32768, 512, 4096
+    # K and V once in bf16, q in and context out in f32, one block-table entry per page, the new row
+    assert bench.algorithmic_bytes(rows, kv_dim, q_dim, False) == 2 * rows * kv_dim * 2 + 2 * q_dim * 4 + 2048 * 4
+    assert bench.algorithmic_bytes(rows, kv_dim, q_dim, True) - bench.algorithmic_bytes(rows, kv_dim, q_dim, False) \
+        == 2 * kv_dim * 2
+    assert bench.HBM_PEAK_GBPS == 8000.0
+
+
+@pytest.mark.gpu
+def test_default_run_prints_one_json_line_with_the_agreed_keys():
+    r = subprocess.run([sys.executable, BENCH, "--steps", "16", "--warmup", "2", "--cpu-seconds", "1"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
+                "scaling", "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 16 and d["warmup"] == 2 and d["higher_is_better"] is False
+    assert d["unit"] == "us/token" and d["vs_baseline"] is None and d["data"] == "synthetic"
+    assert "workload" in d["config"] and "configs[2]" in d["config"]["workload"]
+    rf = d["roofline"]
+    assert rf["bound"] == "hbm" and rf["unit"] == "GB/s" and rf["peak"] == 8000.0
+    assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 1e-3
+    assert abs(rf["achieved"] - rf["bytes_per_launch"] / rf["avg_launch_us"] / 1e3) / rf["achieved"] < 1e-2
+    cb = d["cpu_baseline"]
+    assert cb["kind"] == "port" and cb["unit"] == "us/token" and cb["cores"] >= 1 and cb["value"] > 0
+    assert d["ceiling"]["read_only_launch_us"] > 0
