@@ -63,7 +63,7 @@ def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> 
     return b
 
 
-def bench_restore(skv, torch, np, state, stream):
+def bench_restore(skv, torch, np, state, stream, element="bf16"):
     """Prefix block restore (BASELINE.json configs[3] shapes): the 4096-token shared prefix,
     256 hash blocks of 16 tokens over 36 layers of Qwen3-4B KV (8 kv heads, head_dim 128), is
     matched by chained hash and gathered from the hot cache's page pool into a fresh
@@ -72,11 +72,13 @@ def bench_restore(skv, torch, np, state, stream):
     from saragossa_amd import BlockHash
     qh, kvh, hd, nl, n_tok, bt = 32, 8, 128, 36, 4096, 16
     dev = torch.device("cuda:0")
+    f32 = element == "f32"
+    esize = 4 if f32 else 2
 
     def make(seed):
         out = []
         for i in range(nl):
-            kv = state.full_attention_bf16(n_tok + 16, qh, kvh, hd)
+            kv = (state.full_attention_f32 if f32 else state.full_attention_bf16)(n_tok + 16, qh, kvh, hd)
             kv.set_block_table(np.random.default_rng(seed * 100 + i).permutation(kv.pages())
                                .astype(np.int32))
             out.append(kv)
@@ -135,16 +137,16 @@ def bench_restore(skv, torch, np, state, stream):
         if it >= 3:
             times.append(e0.elapsed_time(e1) * 1e3)
     assert reused == n_tok
-    same = all(np.array_equal(a.read_rows(0, 96)[0], b.read_rows(0, 96)[0]) and
-               np.array_equal(a.read_rows(n_tok - 40, 40)[1], b.read_rows(n_tok - 40, 40)[1])
+    same = all(np.array_equal(a.read_rows_f32(0, 96)[0], b.read_rows_f32(0, 96)[0]) and
+               np.array_equal(a.read_rows_f32(n_tok - 40, 40)[1], b.read_rows_f32(n_tok - 40, 40)[1])
                for a, b in zip(src[::7], dst[::7]))
     if not same:
         raise RuntimeError("restore: restored rows differ from the snapshotted rows")
     times.sort()
     us = times[len(times) // 2]
-    payload = n_tok * nl * 2 * kvh * hd * 2
+    payload = n_tok * nl * 2 * kvh * hd * esize
     out = {"workload": "configs[3]: restore of a 4096-token prefix, 256 blocks x 36 layers, "
-                       "kv8/hd128 bf16 (hash walk on the host included)",
+                       "kv8/hd128 %s (hash walk on the host included)" % element,
            "payload_mib": round(payload / 2 ** 20, 1), "us": round(us, 1),
            "payload_gbps": round(payload / us / 1e3, 1),
            "traffic_gbps": round(2 * payload / us / 1e3, 1),
@@ -655,7 +657,7 @@ def main() -> int:
     del layers, q_all, k_all, v_all
     torch.cuda.empty_cache()
 
-    restore = None if (args.no_restore or args.config != 2) else bench_restore(skv, torch, np, state, stream)
+    restore = None if (args.no_restore or args.config != 2) else bench_restore(skv, torch, np, state, stream, args.element)
     recurrent = None
     if args.config == 2 and not args.no_restore:
         # configs[2]'s 30 linear-attention layers: their recurrent state (conv 96 KiB + ssm 2 MiB
