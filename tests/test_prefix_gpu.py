@@ -19,11 +19,24 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+ELEMENT = "bf16"  # what make_layers builds and check_contents expects; see the `element` fixture
+
+
+@pytest.fixture(params=["bf16", "f32"])
+def element(request):
+    """Runs a test once per element of the cache (the hot cache copies pages of either)."""
+    global ELEMENT
+    ELEMENT = request.param
+    yield request.param
+    ELEMENT = "bf16"
+
+
 def make_layers(state, n_layers, capacity, dims=(32, 8, 128), seed=0, window=0):
     rng = np.random.default_rng(seed)
     layers = []
     for _ in range(n_layers):
-        kv = state.full_attention_bf16(capacity, *dims, window=window)
+        make = state.full_attention_f32 if ELEMENT == "f32" else state.full_attention_bf16
+        kv = make(capacity, *dims, window=window)
         kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
         layers.append(kv)
     return layers
@@ -57,6 +70,10 @@ def check_contents(layers, n, tokens, kv_dim):
     for li, kv in enumerate(layers):
         assert kv.len() == n
         k, v = rows_for(li, range(n), tokens, kv_dim)
+        if ELEMENT == "f32":
+            gk, gv = kv.read_rows_f32()
+            assert np.array_equal(gk, k) and np.array_equal(gv, v), f"layer {li}"
+            continue
         gk, gv = kv.read_rows()
         assert np.array_equal(gk, oracle.f32_to_bf16_bits(k)), f"layer {li} K"
         assert np.array_equal(gv, oracle.f32_to_bf16_bits(v)), f"layer {li} V"
@@ -162,7 +179,7 @@ class SimDecoder(pc.PromptDecoder):
 ])
 def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims, n_layers, bt,
                                                                      prefix, pool_frac,
-                                                                     chunk_blocks, restore_order):
+                                                                     chunk_blocks, restore_order, element):
     kv_dim = dims[1] * dims[2]
     rng = np.random.default_rng(33)
     n_sessions, vocab = 6, 151936
@@ -177,7 +194,7 @@ def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims
     cap = max(len(shared + h + t) for h, t in zip(hist, turns)) + 16
     proto = make_layers(state, n_layers, 16, dims)
     hot = skv.HotCache(state, bt, 10 ** 6, pool_blocks, proto)
-    assert hot.pool_blocks() == pool_blocks and hot.block_bytes() == n_layers * 2 * bt * kv_dim * 2
+    assert hot.pool_blocks() == pool_blocks and hot.block_bytes() == n_layers * 2 * bt * kv_dim * (4 if element == "f32" else 2)
     # oracle run of the same traffic: byte budget = pool size
     ocache = pc.BlockAwarePrefixCache(bt, 10 ** 6, state_bytes=lambda s, m: 1)
     over = lambda extra: len(ocache.entries) + extra > pool_blocks
