@@ -1,7 +1,7 @@
 """BASELINE configs[1]: random-init Qwen3-4B-shaped decoder, chunked prefill over the cache,
 then greedy decode; token ids with the HIP KV path must equal the ids with the CPU oracle's
-KV path, and the caches must hold the same bf16 rows. The default run uses 4 of the 36 layers
-and a 256-token prompt so that the oracle's per-row CPU prefill stays within the suite's time
+KV path, and the caches must hold the same rows. The default run uses 12 of the 36 layers
+and a 1024-token prompt so that the oracle's per-row CPU prefill stays within the suite's time
 budget; SKV_FULL_CONFIG1=1 runs the full 36 layers, 2048-token prompt and 256 steps (several
 minutes of CPU attention)."""
 import os
@@ -25,8 +25,8 @@ def test_config1_greedy_ids_match_oracle(state, hip_cls, ora_cls):
     """ids "fused-pre-kv": decode tokens additionally run the q/k norms and the rotation
     inside the library's fused step (device) against rms_norm_rope_heads_at (CPU).
     "f32-element": both arms keep f32 rows, as the reference does for greedy decoding."""
-    cfg = Config() if FULL else Config(layers=4)
-    n_prompt, n_new, chunk = (2048, 256, 512) if FULL else (256, 48, 96)
+    cfg = Config() if FULL else Config(layers=12)
+    n_prompt, n_new, chunk = (2048, 256, 512) if FULL else (1024, 96, 256)
     w = Weights(cfg, seed=1)
     prompt = [int(t) for t in np.random.default_rng(1).integers(0, cfg.vocab, size=n_prompt)]
     cap = n_prompt + n_new
