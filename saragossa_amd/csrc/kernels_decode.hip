@@ -424,6 +424,35 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         }
     };
 
+    // Keys that no query slot of the workgroup attends (rows at or past the cache's length
+    // after a rollback, ring rows not yet or no longer valid, rows before the window) get zero
+    // probability, but 0 x NaN and 0 x Inf are NaN: their V values are cleared in the
+    // registers as well, so whatever bits such a row holds never reach a context (the
+    // reference never reads those rows, src/decode_resident/kernels.rs:11-88). Only pages
+    // at the edges of the attended range, and ring pages, take the branch.
+    auto mask_v = [&](int pb) __attribute__((always_inline)) {
+        const int first_slot = pb * 16;
+        const bool inside = g.ring_rows == 0 && first_slot >= ws_lo && first_slot + 16 <= lim_hi + 1;
+        if (!inside) {
+            uint32_t keep[2] = {0u, 0u}; // keys 4j, 4j+1 | keys 4j+2, 4j+3: 16 bits each
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int slot = first_slot + j * 4 + i;
+                int pos = slot;
+                if (g.ring_rows > 0)
+                    pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+                if (pos >= ws_lo && pos <= lim_hi) keep[i >> 1] |= 0xffffu << ((i & 1) * 16);
+            }
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                vr[kk].x &= keep[0];
+                vr[kk].z &= keep[0];
+                vr[kk].y &= keep[1];
+                vr[kk].w &= keep[1];
+            }
+        }
+    };
+
     // Steady state is unconditional (the compiler can then wait for exactly the loads it
     // needs); the last page is peeled.
     for (int it = 0; it + 1 < n_it; ++it) {
@@ -435,6 +464,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         short4_t ph, pl;
         softmax_step(s, pb, ph, pl);
         patch_v(pb);
+        mask_v(pb);
         pv(ph, pl);
         load_v<KK>(vr, a, next, kvh, lane);
     }
@@ -445,6 +475,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         short4_t ph, pl;
         softmax_step(s, pb, ph, pl);
         patch_v(pb);
+        mask_v(pb);
         pv(ph, pl);
     }
 

@@ -239,6 +239,25 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
             for (int c = 0; c < NT; ++c) o[c] *= alpha;
         }
     };
+    // Keys that no slot of the tile attends (rows at or past the length after a rollback, ring
+    // rows not valid, rows before the window) have zero probability, but 0 x NaN is NaN: on the
+    // pages at the edges of the attended range (and ring pages) their V values are replaced by
+    // zero in the registers, so the bits of such a row never reach a context (the reference
+    // never reads them, src/decode_resident/kernels.rs:11-88).
+    auto mask_v = [&](int pb, float4_t (&vq)[NT]) {
+        const int slot_a = pb * 16;
+        const bool inside = g.ring_rows == 0 && slot_a >= t_ws_lo && slot_a + 15 <= t_lim_hi;
+        if (inside) return;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int slot = slot_a + j * 4 + k; // this lane's key k
+            int pos = slot;
+            if (g.ring_rows > 0) pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+            const bool live = pos >= t_ws_lo && pos <= t_lim_hi;
+#pragma unroll
+            for (int c = 0; c < NT; ++c) vq[c][k] = live ? vq[c][k] : 0.0f;
+        }
+    };
     // O^T += V^T . P^T, contraction step outermost: consecutive products use different accumulators
     auto accumulate = [&](const float4_t (&vq)[NT], const float (&pv)[4]) {
 #pragma unroll
@@ -251,9 +270,10 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
         // The page after the one being multiplied is already on its way into a second set of
         // registers: without that every wavefront of the device loads, then multiplies, in
         // step, and memory idles half the time.
-        auto consume = [&](int at, const float4_t (&kq)[NT], const float4_t (&vq)[NT]) {
+        auto consume = [&](int at, const float4_t (&kq)[NT], float4_t (&vq)[NT]) {
             float pv[4];
             attend(at, kq, pv);
+            mask_v(at, vq);
             accumulate(vq, pv);
         };
         while (pb < pb1) {
@@ -272,6 +292,7 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
             float pv[4];
             attend(pb, k_a, pv);
             fetch_tile(pb, v_pool, k_a);
+            mask_v(pb, k_a);
             accumulate(k_a, pv);
             if (pb + 4 < pb1) fetch_tile(pb + 4, k_pool, k_a);
         }

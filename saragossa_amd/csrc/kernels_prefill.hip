@@ -65,24 +65,52 @@ __device__ __forceinline__ void fetch_step(uint4 (&stage)[PG][(2 * (P / 32) * 64
 // The K tiles are copied verbatim. The two V tiles of a pair are interleaved in 8-byte
 // halves, unit (kk, h, lane) = {page A's four keys, page B's four keys} of dim tile h, so
 // that one 16-byte read is the 32-key operand of the PV product as it stands.
+//
+// Keys that no query slot of the workgroup attends (rows at or past the cache's length after a
+// rollback, ring rows not valid, rows before every slot's window, the stand-in page past the
+// end of a split) get zero probability, but 0 x NaN is NaN: on the pages at the edges of the
+// attended range [ws_lo, lim_hi] (and on ring pages) their V values are cleared on the way
+// into LDS, so the bits of such a row never reach a context (the reference never reads those
+// rows, src/decode_resident/kernels.rs:11-88).
 template <int P, int PG, int THREADS>
 __device__ __forceinline__ void store_step(const uint4 (&stage)[PG][(2 * (P / 32) * 64 + THREADS - 1) / THREADS], uint4 *buf,
-                                           int tid) {
+                                           int tid, const DecodeArgs &a, int pb0, int step, int n_it, int ws_lo,
+                                           int lim_hi) {
     constexpr int TILE_U4 = (P / 32) * 64;
     constexpr int LOAD_U = (2 * TILE_U4 + THREADS - 1) / THREADS;
     static_assert(PG % 2 == 0, "pages are consumed in pairs");
 #pragma unroll
     for (int pg = 0; pg < PG; ++pg) {
         uint4 *pair = buf + (pg >> 1) * 4 * TILE_U4;
+        const int it = step * PG + pg;
+        const int slot_a = (pb0 + it) * 16; // first cache slot of the page
+        const bool inside = it < n_it && a.g.ring_rows == 0 && slot_a >= ws_lo && slot_a + 15 <= lim_hi;
 #pragma unroll
         for (int u = 0; u < LOAD_U; ++u) {
             const int i = tid + u * THREADS;
             if (2 * TILE_U4 < THREADS && i >= 2 * TILE_U4) continue;
-            const uint4 x = stage[pg][u];
+            uint4 x = stage[pg][u];
             if (i < TILE_U4) {
                 pair[(pg & 1) * TILE_U4 + i] = x;
             } else {
                 const int iv = i - TILE_U4;
+                if (!inside) {
+                    // the unit holds keys 4rq .. 4rq+3 of two dim tiles: (x, y) and (z, w), two keys a word
+                    const int rq = (iv >> 4) & 3;
+                    uint32_t keep[2] = {0u, 0u};
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int slot = slot_a + rq * 4 + r;
+                        int pos = slot;
+                        if (a.g.ring_rows > 0)
+                            pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - a.g.ring_rows + slot;
+                        if (it < n_it && pos >= ws_lo && pos <= lim_hi) keep[r >> 1] |= 0xffffu << ((r & 1) * 16);
+                    }
+                    x.x &= keep[0];
+                    x.z &= keep[0];
+                    x.y &= keep[1];
+                    x.w &= keep[1];
+                }
                 uint2 *dst = reinterpret_cast<uint2 *>(pair + 2 * TILE_U4 + (iv >> 6) * 128 + (iv & 63)) + (pg & 1);
                 dst[0] = make_uint2(x.x, x.y);
                 dst[128] = make_uint2(x.z, x.w); // dim tile 1: 64 units of 16 bytes further
@@ -211,7 +239,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
     uint4 stage[PG][LOAD_U];
     // (a split without pages still reads one valid page, and writes empty partials below)
     fetch_step<P, PG, THREADS>(stage, a, pb0, 0, n_it, kvh, tid);
-    store_step<P, PG, THREADS>(stage, kv_lds, tid);
+    store_step<P, PG, THREADS>(stage, kv_lds, tid, a, pb0, 0, n_it, wg_ws_lo, wg_lim_hi);
     __syncthreads();
 
     for (int step = 0; step < n_steps; ++step) {
@@ -333,7 +361,8 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
             }
         }
       }
-      store_step<P, PG, THREADS>(stage, kv_lds + ((step + 1) & 1) * BUF_U4, tid);
+      store_step<P, PG, THREADS>(stage, kv_lds + ((step + 1) & 1) * BUF_U4, tid, a, pb0, min(step + 1, n_steps - 1),
+                                 n_it, wg_ws_lo, wg_lim_hi);
       __syncthreads();
     }
 
