@@ -32,6 +32,7 @@ extern "C" {
 #define SKV_ERR_DIMENSION 1 /* InferError::Dimension: shapes, overflow at capacity, empty KV/window */
 #define SKV_ERR_CONFIG 2    /* InferError::Config: zero dimension, bad GQA ratio, unsupported option */
 #define SKV_ERR_DEVICE 3    /* InferError::Metal: device/runtime failure, null pointer, wrong element */
+#define SKV_ERR_MEMORY 4    /* InferError::MemoryGuard: an allocation would pass the memory ceiling */
 
 #define SKV_DTYPE_F32 0  /* GpuElement::F32: rows kept as they arrive */
 #define SKV_DTYPE_BF16 1 /* GpuElement::Bf16 */
@@ -50,7 +51,8 @@ typedef struct skv_hot skv_hot;
  * device must be current on the calling thread (the *_host entry points and the create /
  * destroy calls make it current themselves). Two exceptions allocate, after a device
  * synchronisation: a chunked-prefill call whose split partials need more scratch than any
- * call before it on the context (the buffer only grows), and the first attention call of a
+ * call before it on the same context and stream (one buffer per stream, which only grows: calls
+ * on different streams never share partials), and the first attention call of a
  * layer on the plain kernel (RETI_RUST_FLASH_SDPA=0), which creates its score buffer. Host-side bookkeeping (len, ring position)
  * advances when the call returns, before the device has run the work, exactly like the
  * reference's encode-time `len += 1` (src/decode_resident/attention.rs:993); buffers handed
@@ -76,6 +78,21 @@ int32_t skv_flag_flash_sdpa_enabled(void);        /* RETI_RUST_FLASH_SDPA, utils
 int32_t skv_flag_sdpa_2pass_enabled(void);        /* RETI_RUST_SDPA_2PASS, utils.rs:260-263 */
 size_t skv_flag_sdpa_2pass_min_len(void);         /* RETI_RUST_SDPA_2PASS_MIN_LEN, utils.rs:270-278 */
 size_t skv_sdpa_2pass_blocks(size_t len);         /* utils.rs:282-286 */
+/* Rows from which this library splits the context of a decode launch: RETI_RUST_SDPA_2PASS_MIN_LEN
+ * when it is set (the reference's parse, default 2048 when unparsable), else 128. The reference's
+ * own default (2048, utils.rs:270-278) is what skv_flag_sdpa_2pass_min_len reports; it was tuned
+ * for another GPU, and one workgroup per kv head would leave this one idle. */
+size_t skv_effective_split_min_len(void);
+int32_t skv_flag_kv_bf16_sim_konly(void);         /* RETI_RUST_KV_BF16_SIM_KONLY, utils.rs:245-248; honoured by skv_seed */
+int32_t skv_flag_kv_bf16_sim_vonly(void);         /* RETI_RUST_KV_BF16_SIM_VONLY, utils.rs:253-256; honoured by skv_seed */
+/* RETI_RUST_ATTENTION_PAR_THRESHOLD (runtime_flags.rs:641-649, default 128): cache length from
+ * which the CPU path spreads the query heads over threads (src/decoder/attention_ops.rs:926).
+ * The device path has no use for it; a host that keeps a CPU fallback reads it here. */
+size_t skv_flag_attention_par_threshold(void);
+/* RETI_RUST_DECODE_PIPELINE (runtime_flags.rs:309-313, default on): whether the host keeps
+ * several tokens in flight (src/decoder/generation.rs:831). Every *_device entry point only
+ * queues work, so both settings are served; the getter is for the host's loop. */
+int32_t skv_flag_decode_pipeline(void);
 int32_t skv_flag_decode_resident_full(void);      /* RETI_RUST_DECODE_RESIDENT_FULL, runtime_flags.rs:283-286 */
 int32_t skv_flag_decode_resident(void);           /* RETI_RUST_DECODE_RESIDENT, runtime_flags.rs:266-269 */
 int32_t skv_flag_serve_prefix_cache_enabled(void);   /* RETI_SERVE_PREFIX_CACHE, runtime_flags.rs:681-684 */
@@ -96,6 +113,17 @@ size_t skv_window_start(size_t position, size_t window);
  * "capacité KV résidente déborde"). A capacity of 0 means there is nothing to set up. */
 int32_t skv_resident_capacity(size_t prefill_len, size_t max_new_tokens, size_t draft_headroom,
                               size_t *capacity);
+/* The KV part of check_resident_full_decode_allocation (src/decoder/resident/setup.rs:897-917):
+ * sum over the layers of 2 * capacity * kv_dims[i] * elem_bytes (the reference counts
+ * size_of::<f32>() = 4), each product checked, the sum saturating. Returns 1 and writes *bytes,
+ * or 0 when a product overflows ("KV résident déborde"). */
+int32_t skv_resident_kv_bytes(size_t capacity, const size_t *kv_dims, size_t n_layers, size_t elem_bytes,
+                              uint64_t *bytes);
+/* MemoryGuard::projection_with_reserved / projection_over_limit (src/memory_guard.rs:334-362):
+ * projected = current + reserved + requested (saturating), available = limit - (current +
+ * reserved), floored at 0. Returns 1 when projected > limit, else 0. Pure arithmetic. */
+int32_t skv_memory_projection(uint64_t current, uint64_t reserved, uint64_t requested, uint64_t limit,
+                              uint64_t *projected, uint64_t *available);
 /* f32 -> bf16 bits, the reference's formula (src/decode_resident/utils.rs:55-60). Host helper. */
 uint16_t skv_f32_to_bf16_bits(float value);
 
@@ -116,8 +144,11 @@ int32_t skv_ctx_synchronize(skv_ctx *ctx);
 
 /* DecodeResidentState::full_attention_with_element (src/decode_resident/attention.rs:56-108).
  * Rejects a zero dimension and q_heads % kv_heads != 0 with SKV_ERR_CONFIG.
- * `window` > 0 makes the layer a ring buffer that keeps the last `window` rows
- * (rounded up to whole pages); 0 keeps all `capacity` rows in pages.
+ * `window` > 0 makes the layer a ring buffer that keeps the last `window` rows plus
+ * SKV_RING_SLACK_ROWS (environment, default 32) rows behind them, rounded up to whole pages:
+ * the slack is what lets a speculative verify of up to that many rows be rolled back with
+ * skv_truncate (the reference keeps the whole cache and rolls back freely,
+ * src/decoder/attention_cache.rs:72-100); 0 keeps all `capacity` rows in pages.
  * `dtype` is what the pages hold: SKV_DTYPE_BF16 (rows rounded to nearest even at append,
  * pages of kv_heads * P * 32 bytes per tensor, P = head_dim rounded up to a power of two) or
  * SKV_DTYPE_F32 (rows verbatim; pages twice the bytes). head_dim up to 512 in both. Every
@@ -129,6 +160,20 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
 int32_t skv_layer_create_for(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
                              size_t head_dim, int32_t sampled, skv_layer **out);
 void skv_layer_destroy(skv_layer *layer);
+/* Device bytes skv_layer_create will take for these arguments (pools of whole pages, block
+ * table, split partials, staging rows), after the same checks: what a host adds up before it
+ * creates a model's layers, where the reference adds up 2 * capacity * kv_dim * 4 per layer
+ * (check_resident_full_decode_allocation, src/decoder/resident/setup.rs:897-962). A bf16
+ * layer takes about half of an f32 one; a ring layer's size follows its window, not capacity. */
+int32_t skv_layer_bytes(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
+                        size_t window, uint64_t *bytes);
+/* MemoryGuard::check_allocation (src/memory_guard.rs:365-370) against the context's device:
+ * current = device memory in use minus what the context's own arena holds for reuse, limit =
+ * device memory - headroom, further capped by static_cap when that is not 0. SKV_ERR_MEMORY
+ * when current + requested > limit; *available and *projected (either may be null) as in
+ * MemoryProjection. */
+int32_t skv_check_allocation(skv_ctx *ctx, uint64_t requested, uint64_t static_cap, uint64_t headroom,
+                             uint64_t *available, uint64_t *projected);
 
 /* Replace the block table (logical block -> physical page) with a permutation of
  * [0, skv_layer_pages). Only while the layer is empty. No reference counterpart:
@@ -412,7 +457,10 @@ int32_t skv_hot_remember_range(skv_hot *hot, skv_stream stream, const uint8_t se
 /* The hit branch of prefill_prompt_state (src/serve/state.rs:574-584): longest cached
  * chain for `tokens` under `root`, its pages gathered into rows [0, *reused_tokens) of the
  * layers, the last block's recurrent state copied to state_ptrs, each layer's len set to
- * *reused_tokens. *reused_tokens = 0 on a miss (layers untouched). */
+ * *reused_tokens. *reused_tokens = 0 on a miss (layers untouched). The copies of the first
+ * matched blocks are queued while the rest of the chain is still being hashed: an error found
+ * after that (a chain longer than a layer's capacity, state buffers that do not match) leaves
+ * every layer empty (len 0), never with its old length over overwritten rows. */
 int32_t skv_hot_match_restore(skv_hot *hot, skv_stream stream, const uint8_t root[32],
                               const uint64_t *tokens, size_t n_tokens, skv_layer *const *layers,
                               size_t n_layers, void *const *state_ptrs, const size_t *state_bytes,
@@ -430,6 +478,43 @@ uint64_t skv_hot_evictions(const skv_hot *hot);
 uint64_t skv_hot_skipped(const skv_hot *hot);
 int32_t skv_hot_entry(const skv_hot *hot, size_t index, uint8_t session[32], uint8_t hash[32],
                       size_t *tokens, size_t *bytes);
+
+/* ---- the decoder's own whole-prompt cache: prefix_cache_get / prefix_cache_put ------------ */
+
+/* A few whole prompts, most recent first, each with the K/V rows of every layer and the model's
+ * opaque state buffers (final hidden state, recurrent states) as device snapshots
+ * (PrefixCacheEntry, src/decoder/generation.rs:175-188). capacity 0 = disabled: put is a no-op. */
+typedef struct skv_prompt_cache skv_prompt_cache;
+int32_t skv_prompt_cache_create(skv_ctx *ctx, size_t capacity, skv_prompt_cache **out);
+/* capacity = RETI_RUST_PREFIX_CACHE_CAP (default 4), or 0 when RETI_RUST_PREFIX_CACHE=0
+ * (src/runtime_flags.rs:665-678). */
+int32_t skv_prompt_cache_from_runtime_flags(skv_ctx *ctx, skv_prompt_cache **out);
+void skv_prompt_cache_destroy(skv_prompt_cache *cache);
+size_t skv_prompt_cache_len(const skv_prompt_cache *cache);
+size_t skv_prompt_cache_capacity(const skv_prompt_cache *cache);
+size_t skv_prompt_cache_bytes(const skv_prompt_cache *cache);
+/* Entry `index` in recency order (0 = most recent): *n_tokens and, if tokens_out is not null,
+ * its first min(tokens_cap, *n_tokens) tokens. The tests' view of the entries. */
+int32_t skv_prompt_cache_entry(const skv_prompt_cache *cache, size_t index, size_t *n_tokens,
+                               uint64_t *tokens_out, size_t tokens_cap);
+/* prefix_cache_put (generation.rs:3105-3139): a deep copy of rows [0, n_tokens) of every layer
+ * (each layer's len must be n_tokens) and of the n_states state buffers, keyed by the prompt's
+ * tokens; an entry with the same tokens is replaced, the new entry is the most recent, the
+ * least recent ones beyond the capacity are dropped. Async on `stream`; dropping an entry waits
+ * for the device before its memory is freed. */
+int32_t skv_prompt_cache_put(skv_prompt_cache *cache, skv_stream stream, const uint64_t *tokens,
+                             size_t n_tokens, skv_layer *const *layers, size_t n_layers,
+                             const void *const *state_ptrs, const size_t *state_bytes, size_t n_states);
+/* prefix_cache_get (generation.rs:2998-3025) up to the point where the model runs: the longest
+ * entry whose tokens `prompt` starts with (longest_prefix_entry_index, generation.rs:190-204)
+ * becomes the most recent one, its rows are copied into rows [0, *cached_tokens) of the layers
+ * (len set to it), its state buffers into state_ptrs. *cached_tokens = 0 on a miss (layers
+ * untouched). When *cached_tokens < n_prompt the caller extends the layers with the suffix and
+ * puts the whole prompt (generation.rs:3016-3019). Every check precedes the first copy. */
+int32_t skv_prompt_cache_get(skv_prompt_cache *cache, skv_stream stream, const uint64_t *prompt,
+                             size_t n_prompt, skv_layer *const *layers, size_t n_layers,
+                             void *const *state_ptrs, const size_t *state_bytes, size_t n_states,
+                             size_t *cached_tokens);
 
 #ifdef __cplusplus
 }

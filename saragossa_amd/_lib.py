@@ -7,7 +7,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = os.path.join(_HERE, "libsaragossa_kv.so")
 
-OK, ERR_DIMENSION, ERR_CONFIG, ERR_DEVICE = 0, 1, 2, 3
+OK, ERR_DIMENSION, ERR_CONFIG, ERR_DEVICE, ERR_MEMORY = 0, 1, 2, 3, 4
 DTYPE_F32, DTYPE_BF16 = 0, 1
 PAGE_ROWS = 16
 
@@ -30,7 +30,14 @@ class DeviceError(KvError):
     code = ERR_DEVICE
 
 
-_BY_CODE = {ERR_DIMENSION: DimensionError, ERR_CONFIG: ConfigError, ERR_DEVICE: DeviceError}
+class MemoryGuardError(KvError):
+    """InferError::MemoryGuard (src/error.rs:66-68)."""
+
+    code = ERR_MEMORY
+
+
+_BY_CODE = {ERR_DIMENSION: DimensionError, ERR_CONFIG: ConfigError, ERR_DEVICE: DeviceError,
+            ERR_MEMORY: MemoryGuardError}
 
 _lib = None
 
@@ -47,6 +54,17 @@ SIGNATURES = {
     "skv_flag_sdpa_2pass_enabled": (_i32, []),
     "skv_flag_sdpa_2pass_min_len": (_sz, []),
     "skv_sdpa_2pass_blocks": (_sz, [_sz]),
+    "skv_effective_split_min_len": (_sz, []),
+    "skv_flag_kv_bf16_sim_konly": (_i32, []),
+    "skv_flag_kv_bf16_sim_vonly": (_i32, []),
+    "skv_flag_attention_par_threshold": (_sz, []),
+    "skv_flag_decode_pipeline": (_i32, []),
+    "skv_resident_kv_bytes": (_i32, [_sz, _vp, _sz, _sz, C.POINTER(C.c_uint64)]),
+    "skv_memory_projection": (_i32, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64,
+                                     C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "skv_layer_bytes": (_i32, [_sz, _sz, _sz, _sz, _i32, _sz, C.POINTER(C.c_uint64)]),
+    "skv_check_allocation": (_i32, [_vp, C.c_uint64, C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64),
+                                    C.POINTER(C.c_uint64)]),
     "skv_flag_decode_resident_full": (_i32, []),
     "skv_flag_decode_resident": (_i32, []),
     "skv_flag_serve_prefix_cache_enabled": (_i32, []),
@@ -146,6 +164,15 @@ SIGNATURES = {
     "skv_hot_evictions": (C.c_uint64, [_vp]),
     "skv_hot_skipped": (C.c_uint64, [_vp]),
     "skv_hot_entry": (_i32, [_vp, _sz, _vp, _vp, C.POINTER(_sz), C.POINTER(_sz)]),
+    "skv_prompt_cache_create": (_i32, [_vp, _sz, C.POINTER(_vp)]),
+    "skv_prompt_cache_from_runtime_flags": (_i32, [_vp, C.POINTER(_vp)]),
+    "skv_prompt_cache_destroy": (None, [_vp]),
+    "skv_prompt_cache_len": (_sz, [_vp]),
+    "skv_prompt_cache_capacity": (_sz, [_vp]),
+    "skv_prompt_cache_bytes": (_sz, [_vp]),
+    "skv_prompt_cache_entry": (_i32, [_vp, _sz, C.POINTER(_sz), _vp, _sz]),
+    "skv_prompt_cache_put": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz]),
+    "skv_prompt_cache_get": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz, C.POINTER(_sz)]),
 }
 
 

@@ -76,8 +76,9 @@ template <typename T> struct Once {
     }
 };
 
-Once<int> f_flash, f_2pass, f_res_full, f_res, f_serve_prefix, f_prefix, f_kv_bf16;
-Once<size_t> f_2pass_min, f_block_tokens, f_cache_blocks, f_per_session, f_prefix_cap, f_chunk;
+Once<int> f_flash, f_2pass, f_res_full, f_res, f_serve_prefix, f_prefix, f_kv_bf16, f_sim_k, f_sim_v, f_pipeline;
+Once<size_t> f_2pass_min, f_block_tokens, f_cache_blocks, f_per_session, f_prefix_cap, f_chunk, f_par_threshold,
+    f_split_min;
 
 } // namespace
 
@@ -114,6 +115,28 @@ size_t skv_flag_sdpa_2pass_min_len(void) {
     return f_2pass_min.get([] {
         return parse_usize(std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN"), false).value_or(2048);
     });
+}
+size_t skv_effective_split_min_len(void) {
+    // The reference's default switch-over (2048 rows, src/decode_resident/utils.rs:270-278) was
+    // tuned for Apple GPUs; an explicit RETI_RUST_SDPA_2PASS_MIN_LEN is honoured as it is, the
+    // default here is 128 because one workgroup per kv head leaves most compute units idle.
+    return f_split_min.get([] {
+        const char *raw = std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN");
+        return raw ? parse_usize(raw, false).value_or(2048) : (size_t)128;
+    });
+}
+int32_t skv_flag_kv_bf16_sim_konly(void) {
+    return f_sim_k.get([] { return (int)env_flag("RETI_RUST_KV_BF16_SIM_KONLY", false); });
+}
+int32_t skv_flag_kv_bf16_sim_vonly(void) {
+    return f_sim_v.get([] { return (int)env_flag("RETI_RUST_KV_BF16_SIM_VONLY", false); });
+}
+size_t skv_flag_attention_par_threshold(void) {
+    return f_par_threshold.get(
+        [] { return parse_usize(std::getenv("RETI_RUST_ATTENTION_PAR_THRESHOLD"), true).value_or(128); });
+}
+int32_t skv_flag_decode_pipeline(void) {
+    return f_pipeline.get([] { return (int)env_flag("RETI_RUST_DECODE_PIPELINE", true); });
 }
 size_t skv_sdpa_2pass_blocks(size_t len) {
     size_t raw = std::max<size_t>(len / 128, 1);
@@ -190,6 +213,35 @@ int32_t skv_resident_capacity(size_t prefill_len, size_t max_new_tokens, size_t 
         return 0;
     *capacity = b;
     return 1;
+}
+
+int32_t skv_resident_kv_bytes(size_t capacity, const size_t *kv_dims, size_t n_layers, size_t elem_bytes,
+                              uint64_t *bytes) {
+    // checked_bytes(&[2, capacity, kv_dim], size_of::<f32>()) summed with saturating_add
+    // (src/decoder/resident/setup.rs:906-917); an overflowing product is the reference's
+    // "KV résident déborde"
+    if (!bytes || (n_layers && !kv_dims)) return 0;
+    uint64_t total = 0;
+    for (size_t i = 0; i < n_layers; ++i) {
+        uint64_t b = 2;
+        if (__builtin_mul_overflow(b, (uint64_t)capacity, &b) || __builtin_mul_overflow(b, (uint64_t)kv_dims[i], &b) ||
+            __builtin_mul_overflow(b, (uint64_t)elem_bytes, &b))
+            return 0;
+        total = total > UINT64_MAX - b ? UINT64_MAX : total + b;
+    }
+    *bytes = total;
+    return 1;
+}
+
+int32_t skv_memory_projection(uint64_t current, uint64_t reserved, uint64_t requested, uint64_t limit,
+                              uint64_t *projected, uint64_t *available) {
+    // projection_with_reserved + projection_over_limit (src/memory_guard.rs:334-362)
+    auto sat = [](uint64_t a, uint64_t b) { return a > UINT64_MAX - b ? UINT64_MAX : a + b; };
+    const uint64_t before = sat(current, reserved);
+    const uint64_t proj = sat(before, requested);
+    if (projected) *projected = proj;
+    if (available) *available = limit > before ? limit - before : 0;
+    return proj > limit ? 1 : 0;
 }
 
 uint16_t skv_f32_to_bf16_bits(float value) {

@@ -14,8 +14,10 @@ using skv::Geom;
 struct skv_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
-    void *mq_scratch = nullptr; // split-K partials of multi-query launches, grown on demand
-    size_t mq_bytes = 0;
+    // Split-K partials of multi-query launches (chunked prefill), one buffer per stream the
+    // context has seen such a launch on, grown on demand: launches on one stream are ordered by
+    // it, launches on different streams never share a buffer. Guarded by arena_mu.
+    std::map<hipStream_t, std::pair<void *, size_t>> mq_scratch;
     // Device buffers of destroyed layers, kept for the next layer that needs about as much:
     // the stand-in for the arena DecodeResidentState leases its buffers from
     // (src/decode_resident/arena.rs:116-211). A server creates and drops one cache per layer

@@ -64,9 +64,9 @@ void arena_put(skv_ctx *ctx, void *ptr, size_t bytes) {
 // Frees what the context holds on the device; the caller has synchronised the device.
 static void ctx_drain(skv_ctx *ctx) {
     std::lock_guard<std::mutex> lk(ctx->arena_mu);
-    if (ctx->mq_scratch) (void)hipFree(ctx->mq_scratch);
-    ctx->mq_scratch = nullptr;
-    ctx->mq_bytes = 0;
+    for (auto &kv : ctx->mq_scratch)
+        if (kv.second.first) (void)hipFree(kv.second.first);
+    ctx->mq_scratch.clear();
     for (auto &kv : ctx->arena_free) (void)hipFree(kv.second);
     ctx->arena_free.clear();
     ctx->arena_bytes = 0;
@@ -75,7 +75,7 @@ static void ctx_drain(skv_ctx *ctx) {
 void ctx_release(skv_ctx *ctx) {
     if (ctx->refs.fetch_sub(1, std::memory_order_acq_rel) != 1) return;
     // a layer that outlived skv_ctx_destroy may have grown the multi-query scratch again
-    if (ctx->mq_scratch) {
+    if (!ctx->mq_scratch.empty()) {
         (void)hipSetDevice(ctx->device);
         (void)hipDeviceSynchronize();
         ctx_drain(ctx);
@@ -121,11 +121,7 @@ const Tuning &tuning() {
     thread_local uint64_t seen = 0;
     const uint64_t epoch = skv_internal_flags_epoch();
     if (epoch != seen) {
-        // The reference's default switch-over (2048 rows, src/decode_resident/utils.rs:270-278)
-        // was tuned for Apple GPUs; an explicit RETI_RUST_SDPA_2PASS_MIN_LEN is honoured as
-        // is, the default here is 128 because a single workgroup per kv head leaves 250 of
-        // the 256 compute units idle.
-        t.split_min_len = std::getenv("RETI_RUST_SDPA_2PASS_MIN_LEN") ? skv_flag_sdpa_2pass_min_len() : 128;
+        t.split_min_len = skv_effective_split_min_len();
         t.target_wgs = std::max<size_t>(env_usize("SKV_DECODE_WGS", 256), 1);
         t.min_pages = env_usize("SKV_DECODE_MIN_PAGES", 0);
         t.forced_waves = env_usize("SKV_DECODE_WAVES", 0);
@@ -241,20 +237,27 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
 
 // Split partials of a multi-query launch live in the context's scratch, grown on demand:
 // [kv_heads][n_sets][n_queries * gqa] of (o[head_dim], m, l).
-int32_t multi_query_partials(skv_layer *L, size_t n_sets, size_t n_queries, DecodeArgs &a) {
+int32_t multi_query_partials(skv_layer *L, hipStream_t s, size_t n_sets, size_t n_queries, DecodeArgs &a) {
     const Geom &g = L->g;
     const size_t n_part = (size_t)g.kv_heads * n_sets * n_queries * g.gqa;
     const size_t need = n_part * ((size_t)g.head_dim + 2) * sizeof(float);
     skv_ctx *c = L->ctx;
-    if (c->mq_bytes < need) {
-        SKV_HIP(hipDeviceSynchronize());
-        if (c->mq_scratch) SKV_HIP(hipFree(c->mq_scratch));
-        c->mq_scratch = nullptr;
-        c->mq_bytes = 0;
-        SKV_HIP(hipMalloc(&c->mq_scratch, need));
-        c->mq_bytes = need;
+    void *buf = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(c->arena_mu);
+        auto &slot = c->mq_scratch[s];
+        if (slot.second < need) {
+            // work queued on the stream may still read the old buffer
+            SKV_HIP(hipStreamSynchronize(s));
+            if (slot.first) SKV_HIP(hipFree(slot.first));
+            slot = {nullptr, 0};
+            void *p = nullptr;
+            SKV_HIP(hipMalloc(&p, need));
+            slot = {p, need};
+        }
+        buf = slot.first;
     }
-    a.part_o = reinterpret_cast<float *>(c->mq_scratch);
+    a.part_o = reinterpret_cast<float *>(buf);
     a.part_m = a.part_o + n_part * g.head_dim;
     a.part_l = a.part_m + n_part;
     return SKV_OK;
@@ -299,7 +302,7 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
             a.splits = (int)std::min<size_t>((size_t)a.splits, want);
             a.splits_total = a.splits;
             if (a.splits > 1) {
-                int32_t rc2 = multi_query_partials(L, (size_t)a.splits, n_queries, a);
+                int32_t rc2 = multi_query_partials(L, s, (size_t)a.splits, n_queries, a);
                 if (rc2) return rc2;
             }
         }
@@ -366,7 +369,7 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
         a.splits = (int)std::min<size_t>((size_t)a.splits, want);
         a.splits_total = a.splits;
         if (a.splits > 1) {
-            int32_t rc2 = multi_query_partials(L, (size_t)a.splits, n_queries, a);
+            int32_t rc2 = multi_query_partials(L, s, (size_t)a.splits, n_queries, a);
             if (rc2) return rc2;
         }
     }
@@ -485,10 +488,24 @@ void skv_layer_destroy(skv_layer *L) {
     delete L;
 }
 
-int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
-                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) try {
-    if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_layer_create: pointeur nul");
-    *out = nullptr;
+// Shape checks of full_attention_with_element (src/decode_resident/attention.rs:56-108) and
+// the geometry, page count and buffer sizes that follow from them; shared by the factory and
+// by skv_layer_bytes so that the budget figure is the factory's own arithmetic.
+struct LayerPlan {
+    Geom g{};
+    int n_pages = 0;
+    int max_splits = 1;
+    size_t pool_bytes = 0, table_bytes = 0, part_o_bytes = 0, part_ml_bytes = 0, q_bytes = 0, kv_stage_bytes = 0;
+    size_t total() const {
+        // every buffer is its own allocation, rounded up by the allocator to 256 bytes at least
+        auto r = [](size_t b) { return (std::max<size_t>(b, 256) + 255) / 256 * 256; };
+        return 2 * r(pool_bytes) + r(table_bytes) + r(part_o_bytes) + 2 * r(part_ml_bytes) + 2 * r(q_bytes) +
+               r(kv_stage_bytes);
+    }
+};
+
+static int32_t plan_layer(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
+                          size_t window, LayerPlan &p) {
     if (capacity == 0 || q_heads == 0 || kv_heads == 0 || head_dim == 0)
         return fail(SKV_ERR_CONFIG, "FullAttentionMetalState: dimension nulle");
     if (q_heads % kv_heads != 0)
@@ -499,15 +516,9 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     const bool f32 = dtype == SKV_DTYPE_F32;
     const int P = padded_head_dim(head_dim);
     if (P == 0) return fail(SKV_ERR_CONFIG, "head_dim > 512 non supporté");
-    if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096)
+    if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096 || window > (size_t)1 << 30)
         return fail(SKV_ERR_CONFIG, "capacité KV déborde");
-    SKV_HIP(hipSetDevice(ctx->device));
-
-    skv_layer *L = new skv_layer();
-    L->ctx = ctx;
-    L->capacity = capacity;
-    L->window = window;
-    Geom &g = L->g;
+    Geom &g = p.g;
     g.q_heads = (int)q_heads;
     g.kv_heads = (int)kv_heads;
     g.head_dim = (int)head_dim;
@@ -518,15 +529,94 @@ int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t k
     g.page_elems = (int)kv_heads * g.tile_elems;
     size_t rows = capacity;
     if (window > 0) {
-        const size_t ring = (window + 15) / 16 * 16;
+        // The ring keeps the window plus some rows behind it, so that the rows a speculative
+        // verify appended can be rolled back (truncate) without the ring having overwritten
+        // what the next query attends: the reference keeps the whole cache and rolls back
+        // freely (src/decoder/attention_cache.rs:72-100). A ring never needs more rows than
+        // the capacity.
+        const size_t slack = env_usize("SKV_RING_SLACK_ROWS", 32);
+        size_t ring = (window + slack + 15) / 16 * 16;
+        ring = std::min(ring, (capacity + 15) / 16 * 16);
         g.ring_rows = (int)ring;
         rows = ring;
     }
-    L->n_pages = (int)((rows + 15) / 16);
-    const size_t pool_bytes = (size_t)L->n_pages * g.page_elems * sizeof(uint16_t);
+    p.n_pages = (int)((rows + 15) / 16);
+    p.pool_bytes = (size_t)p.n_pages * g.page_elems * sizeof(uint16_t);
+    p.max_splits = std::min(decode_max_splits(), std::max(1, p.n_pages));
+    const size_t n_part = (size_t)kv_heads * p.max_splits * g.gqa;
+    p.table_bytes = (size_t)p.n_pages * sizeof(int32_t);
+    p.part_o_bytes = n_part * head_dim * sizeof(float);
+    p.part_ml_bytes = n_part * sizeof(float);
+    p.q_bytes = q_heads * head_dim * sizeof(float);
+    p.kv_stage_bytes = 2 * kv_heads * head_dim * sizeof(float);
+    return SKV_OK;
+}
+
+int32_t skv_layer_bytes(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
+                        size_t window, uint64_t *bytes) try {
+    if (!bytes) return fail(SKV_ERR_DEVICE, "skv_layer_bytes: pointeur nul");
+    LayerPlan p;
+    int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, p);
+    if (rc) return rc;
+    *bytes = (uint64_t)p.total();
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_check_allocation(skv_ctx *ctx, uint64_t requested, uint64_t static_cap, uint64_t headroom,
+                             uint64_t *available, uint64_t *projected) try {
+    if (!ctx) return fail(SKV_ERR_DEVICE, "skv_check_allocation: ctx nul");
+    SKV_HIP(hipSetDevice(ctx->device));
+    size_t free_b = 0, total_b = 0;
+    SKV_HIP(hipMemGetInfo(&free_b, &total_b));
+    // effective_limit: the smallest of the caps that are set (src/memory_guard.rs:109-127); the
+    // device's memory minus the headroom stands where the host's memory stands there
+    uint64_t limit = (uint64_t)total_b > headroom ? (uint64_t)total_b - headroom : 0;
+    if (static_cap) limit = std::min(limit, static_cap);
+    // what the context's arena holds is free for the next layers of the same context
+    uint64_t held = 0;
+    {
+        std::lock_guard<std::mutex> lk(ctx->arena_mu);
+        held = ctx->arena_bytes;
+    }
+    const uint64_t used = (uint64_t)(total_b - free_b);
+    const uint64_t current = used > held ? used - held : 0;
+    uint64_t proj = 0, avail = 0;
+    const int32_t over = skv_memory_projection(current, 0, requested, limit, &proj, &avail);
+    if (available) *available = avail;
+    if (projected) *projected = proj;
+    if (over)
+        return fail(SKV_ERR_MEMORY, "garde mémoire: demande " + std::to_string(requested) + " o, projection " +
+                                        std::to_string(proj) + " o > plafond " + std::to_string(limit) +
+                                        " o (disponible " + std::to_string(avail) + " o)");
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
+                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) try {
+    if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_layer_create: pointeur nul");
+    *out = nullptr;
+    LayerPlan plan;
+    {
+        int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, plan);
+        if (rc) return rc;
+    }
+    SKV_HIP(hipSetDevice(ctx->device));
+
+    skv_layer *L = new skv_layer();
+    L->ctx = ctx;
+    L->capacity = capacity;
+    L->window = window;
+    L->g = plan.g;
+    const Geom &g = L->g;
+    L->n_pages = plan.n_pages;
+    const size_t pool_bytes = plan.pool_bytes;
     const size_t q_dim = q_heads * head_dim;
     const size_t kv_dim = kv_heads * head_dim;
-    L->max_splits = std::min(decode_max_splits(), std::max(1, L->n_pages));
+    L->max_splits = plan.max_splits;
     const size_t n_part = (size_t)kv_heads * L->max_splits * g.gqa;
 
     hipError_t e = hipSuccess;
@@ -635,6 +725,19 @@ int32_t skv_seed(skv_layer *L, const float *keys, const float *values, size_t n_
     L->floor_pos = 0;
     if (n_rows == 0) return SKV_OK;
     hipStream_t s = L->ctx->stream;
+    // RETI_RUST_KV_BF16_SIM_KONLY / _VONLY (src/decode_resident/attention.rs:573-585): on an
+    // f32 cache the seed keeps K alone, or else V alone, at bf16 precision (still stored as f32)
+    std::vector<float> rounded;
+    if (L->g.f32 && (skv_flag_kv_bf16_sim_konly() || skv_flag_kv_bf16_sim_vonly())) {
+        const bool k_only = skv_flag_kv_bf16_sim_konly() != 0; // K wins when both are set, as in the match
+        const float *src = k_only ? keys : values;
+        rounded.resize(expected);
+        for (size_t i = 0; i < expected; ++i) {
+            const uint32_t b = (uint32_t)skv_f32_to_bf16_bits(src[i]) << 16;
+            std::memcpy(&rounded[i], &b, sizeof(float));
+        }
+        (k_only ? keys : values) = rounded.data();
+    }
     float *stage = nullptr;
     SKV_HIP(hipMalloc((void **)&stage, 2 * expected * sizeof(float)));
     hipError_t e = hipMemcpyAsync(stage, keys, expected * sizeof(float), hipMemcpyHostToDevice, s);
@@ -786,7 +889,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
         a1.splits = s1;
         a1.split_base = 0;
         a1.splits_total = total;
-        int32_t rc = multi_query_partials(L, (size_t)total, c, a1);
+        int32_t rc = multi_query_partials(L, s, (size_t)total, c, a1);
         if (rc) return rc;
         SKV_HIP(launch_chunk(a1));
     }
@@ -799,7 +902,7 @@ static int32_t ring_chunk(skv_layer *L, hipStream_t s, const float *q, const flo
     a3.split_base = s1;
     a3.splits_total = total;
     if (total > 1) {
-        rc = multi_query_partials(L, (size_t)total, c, a3);
+        rc = multi_query_partials(L, s, (size_t)total, c, a3);
         if (rc) return rc;
     }
     SKV_HIP(launch_chunk(a3));
@@ -1204,7 +1307,7 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
             return fail(SKV_ERR_DEVICE, "decode_step_batch: pointeur nul (séquence " + std::to_string(i) + ")");
         const Geom &g = L->g, &g0 = seqs[0]->g;
         if (g.q_heads != g0.q_heads || g.kv_heads != g0.kv_heads || g.head_dim != g0.head_dim ||
-            g.ring_rows != g0.ring_rows || g.f32 != g0.f32 || L->window != seqs[0]->window ||
+            (g.ring_rows > 0) != (g0.ring_rows > 0) || g.f32 != g0.f32 || L->window != seqs[0]->window ||
             L->ctx != seqs[0]->ctx)
             return fail(SKV_ERR_DIMENSION, "decode_step_batch: la séquence " + std::to_string(i) +
                                                " n'a pas la géométrie de la séquence 0");

@@ -785,11 +785,22 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
     size_t done_blocks = 0; // blocks whose copies have been queued
     size_t batch = any_ring ? (size_t)-1 : 16;
     const size_t bt = h->index->block_tokens();
+    // Once the first batch of copies is queued the layers' rows are being overwritten: an
+    // error after that point leaves every layer empty (len 0) rather than with its old length
+    // over rows that are no longer its own.
+    auto fail_emptied = [&](int32_t code) {
+        if (done_blocks > 0)
+            for (size_t l = 0; l < n_layers; ++l) {
+                layers[l]->len = 0;
+                layers[l]->floor_pos = 0;
+            }
+        return code;
+    };
     for (;;) {
         const size_t got = h->index->match_more(&walk, root, tokens, n_tokens, batch, &hit, &chain);
         if (chain.size() * bt > min_capacity)
-            return fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(chain.size() * bt) +
-                                               " > capacité " + std::to_string(min_capacity));
+            return fail_emptied(fail(SKV_ERR_DIMENSION, "seed KV " + std::to_string(chain.size() * bt) +
+                                                            " > capacité " + std::to_string(min_capacity)));
         if (got == 0) break;
         if (!any_ring) {
             pages.clear();
@@ -803,8 +814,8 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
             }
             rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(),
                             pages.size(), nullptr, false, as_stream(stream));
-            if (rc) return rc;
             done_blocks = chain.size();
+            if (rc) return fail_emptied(rc);
             // a copy of b pages takes about 2.4 times as long as hashing b blocks, so the next
             // batch may be that much larger without the queue running dry
             batch = std::min<size_t>(batch * 5 / 2, COPY_MAX_PAGES);
@@ -812,6 +823,9 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
         if (!walk.alive) break;
     }
     if (chain.empty()) return SKV_OK;
+    const HotEntry &last = h->entries.at(chain.back());
+    if (n_states && !last.state)
+        return fail_emptied(fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=0 couches=" + std::to_string(n_states)));
     const size_t reused = hit.tokens;
     std::vector<uint32_t> first_page(n_layers, 0);
     if (any_ring) {
@@ -829,13 +843,12 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
         }
         rc = copy_pages(h->layout, h->pool, layers, n_layers, pages.data(), slots.data(), pages.size(),
                         first_page.data(), false, as_stream(stream));
-        if (rc) return rc;
+        done_blocks = chain.size();
+        if (rc) return fail_emptied(rc);
     }
-    const HotEntry &last = h->entries.at(chain.back());
     if (n_states) {
-        if (!last.state) return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=0 couches=" + std::to_string(n_states));
         rc = skv_state_restore(h->ctx, stream, last.state, state_ptrs, state_bytes, n_states);
-        if (rc) return rc;
+        if (rc) return fail_emptied(rc);
     }
     for (size_t l = 0; l < n_layers; ++l) {
         skv_layer *L = layers[l];
@@ -844,6 +857,179 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
     }
     *reused_tokens = reused;
     if (hash_out) std::memcpy(hash_out, hit.hash, 32);
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+// ---- the decoder's own whole-prompt cache ---------------------------------------------------
+// prefix_cache_get / prefix_cache_put (src/decoder/generation.rs:2998-3025, 3105-3139): a few
+// whole prompts (RETI_RUST_PREFIX_CACHE_CAP, default 4), newest first, each with the K/V rows of
+// every layer and the model's opaque state buffers (final hidden state, recurrent states); a
+// request whose prompt starts with a cached prompt resumes from the longest such entry. An
+// entry here is a block snapshot of the prompt's pages plus a state snapshot; a hit copies them
+// into the caller's layers, so what the caller then appends never touches the entry (the
+// reference clones for the same reason, generation.rs:3009).
+} // extern "C"
+
+struct PromptEntry {
+    std::vector<uint64_t> tokens;
+    skv_snapshot *pages = nullptr;
+    skv_snapshot *state = nullptr;
+    size_t bytes = 0;
+};
+
+struct skv_prompt_cache {
+    CtxRef ctx;
+    size_t capacity = 0;
+    std::vector<PromptEntry> entries; // index 0 = most recent
+};
+
+static void prompt_entry_free(PromptEntry &e) {
+    skv_snapshot_free(e.pages);
+    skv_snapshot_free(e.state);
+    e.pages = e.state = nullptr;
+}
+
+// longest_prefix_entry_index (src/decoder/generation.rs:190-204): the first of the longest
+// entries whose tokens the prompt starts with; -1 = none (an empty entry never matches).
+static long longest_prefix_entry_index(const std::vector<PromptEntry> &entries, const uint64_t *prompt, size_t n) {
+    long best = -1;
+    size_t best_len = 0;
+    for (size_t i = 0; i < entries.size(); ++i) {
+        const std::vector<uint64_t> &t = entries[i].tokens;
+        if (t.size() > best_len && t.size() <= n && std::equal(t.begin(), t.end(), prompt)) {
+            best = (long)i;
+            best_len = t.size();
+        }
+    }
+    return best;
+}
+
+extern "C" {
+
+int32_t skv_prompt_cache_create(skv_ctx *ctx, size_t capacity, skv_prompt_cache **out) try {
+    if (!ctx || !out) return fail(SKV_ERR_DEVICE, "prompt_cache_create: pointeur nul");
+    skv_prompt_cache *c = new skv_prompt_cache();
+    c->ctx = ctx;
+    c->capacity = capacity;
+    *out = c;
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_prompt_cache_from_runtime_flags(skv_ctx *ctx, skv_prompt_cache **out) try {
+    // RETI_RUST_PREFIX_CACHE=0 switches the cache off (generation.rs:2781-2784): capacity 0
+    return skv_prompt_cache_create(ctx, skv_flag_prefix_cache_enabled() ? skv_flag_prefix_cache_capacity() : 0, out);
+} catch (...) {
+    return skv::fail_exception();
+}
+
+void skv_prompt_cache_destroy(skv_prompt_cache *c) {
+    if (!c) return;
+    for (PromptEntry &e : c->entries) prompt_entry_free(e);
+    delete c;
+}
+
+size_t skv_prompt_cache_len(const skv_prompt_cache *c) { return c ? c->entries.size() : 0; }
+size_t skv_prompt_cache_capacity(const skv_prompt_cache *c) { return c ? c->capacity : 0; }
+size_t skv_prompt_cache_bytes(const skv_prompt_cache *c) {
+    size_t b = 0;
+    if (c)
+        for (const PromptEntry &e : c->entries) b += e.bytes;
+    return b;
+}
+
+int32_t skv_prompt_cache_entry(const skv_prompt_cache *c, size_t index, size_t *n_tokens, uint64_t *tokens_out,
+                               size_t tokens_cap) try {
+    if (!c || !n_tokens) return fail(SKV_ERR_DEVICE, "prompt_cache_entry: pointeur nul");
+    if (index >= c->entries.size()) return fail(SKV_ERR_DIMENSION, "prompt_cache_entry: indice hors plage");
+    const std::vector<uint64_t> &t = c->entries[index].tokens;
+    *n_tokens = t.size();
+    if (tokens_out) std::copy(t.begin(), t.begin() + std::min(tokens_cap, t.size()), tokens_out);
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_prompt_cache_put(skv_prompt_cache *c, skv_stream stream, const uint64_t *tokens, size_t n_tokens,
+                             skv_layer *const *layers, size_t n_layers, const void *const *state_ptrs,
+                             const size_t *state_bytes, size_t n_states) try {
+    if (!c || (n_tokens && !tokens)) return fail(SKV_ERR_DEVICE, "prompt_cache_put: pointeur nul");
+    if (c->capacity == 0) return SKV_OK;
+    int32_t rc = check_layers(c->ctx, layers, n_layers);
+    if (rc) return rc;
+    for (size_t l = 0; l < n_layers; ++l)
+        if (layers[l]->len != n_tokens)
+            return fail(SKV_ERR_DIMENSION, "prompt_cache_put: la couche " + std::to_string(l) + " tient " +
+                                               std::to_string(layers[l]->len) + " lignes pour un prompt de " +
+                                               std::to_string(n_tokens));
+    // the snapshots first: a failure leaves the cache as it was
+    PromptEntry e;
+    e.tokens.assign(tokens, tokens + n_tokens);
+    std::vector<size_t> blocks((n_tokens + 15) / 16);
+    for (size_t i = 0; i < blocks.size(); ++i) blocks[i] = i;
+    rc = skv_snapshot_blocks(c->ctx, stream, layers, n_layers, blocks.data(), blocks.size(), &e.pages);
+    if (rc) return rc;
+    rc = skv_state_snapshot(c->ctx, stream, state_ptrs, state_bytes, n_states, &e.state);
+    if (rc) {
+        prompt_entry_free(e);
+        return rc;
+    }
+    e.bytes = skv_snapshot_bytes(e.pages) + skv_snapshot_bytes(e.state);
+    for (size_t i = 0; i < c->entries.size(); ++i) {
+        if (c->entries[i].tokens == e.tokens) {
+            prompt_entry_free(c->entries[i]);
+            c->entries.erase(c->entries.begin() + (long)i);
+            break;
+        }
+    }
+    c->entries.insert(c->entries.begin(), std::move(e));
+    while (c->entries.size() > c->capacity) {
+        prompt_entry_free(c->entries.back());
+        c->entries.pop_back();
+    }
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_prompt_cache_get(skv_prompt_cache *c, skv_stream stream, const uint64_t *prompt, size_t n_prompt,
+                             skv_layer *const *layers, size_t n_layers, void *const *state_ptrs,
+                             const size_t *state_bytes, size_t n_states, size_t *cached_tokens) try {
+    if (!c || !cached_tokens || (n_prompt && !prompt)) return fail(SKV_ERR_DEVICE, "prompt_cache_get: pointeur nul");
+    *cached_tokens = 0;
+    const long index = longest_prefix_entry_index(c->entries, prompt, n_prompt);
+    if (index < 0) return SKV_OK;
+    int32_t rc = check_layers(c->ctx, layers, n_layers);
+    if (rc) return rc;
+    const PromptEntry &hit = c->entries[(size_t)index];
+    const size_t cached = hit.tokens.size();
+    // every check before the first copy is queued: a failure leaves the layers untouched
+    for (size_t l = 0; l < n_layers; ++l)
+        if (layers[l]->capacity < cached)
+            return fail(SKV_ERR_DIMENSION, "prompt_cache_get: capacité " + std::to_string(layers[l]->capacity) +
+                                               " < préfixe en cache " + std::to_string(cached));
+    if (hit.state && n_states != hit.state->sizes.size())
+        return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=" + std::to_string(hit.state->sizes.size()) +
+                                           " couches=" + std::to_string(n_states));
+    for (size_t i = 0; i < n_states; ++i)
+        if (!state_ptrs || !state_bytes || state_bytes[i] != hit.state->sizes[i])
+            return fail(SKV_ERR_DIMENSION, "prompt_cache_get: taille du tampon d'état " + std::to_string(i) + " différente");
+    std::vector<size_t> blocks(hit.pages ? hit.pages->n_pages : 0);
+    for (size_t i = 0; i < blocks.size(); ++i) blocks[i] = i;
+    rc = skv_restore_blocks(c->ctx, stream, hit.pages, layers, n_layers, blocks.data(), blocks.size());
+    if (rc) return rc;
+    rc = skv_state_restore(c->ctx, stream, hit.state, state_ptrs, state_bytes, n_states);
+    if (rc) return rc;
+    for (size_t l = 0; l < n_layers; ++l) {
+        layers[l]->len = cached;
+        layers[l]->floor_pos = 0;
+    }
+    // the hit becomes the most recent entry (generation.rs:3007-3012)
+    if (index > 0) std::rotate(c->entries.begin(), c->entries.begin() + index, c->entries.begin() + index + 1);
+    *cached_tokens = cached;
     return SKV_OK;
 } catch (...) {
     return skv::fail_exception();

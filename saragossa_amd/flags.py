@@ -31,6 +31,32 @@ def sdpa_2pass_blocks(n: int) -> int:
     return lib().skv_sdpa_2pass_blocks(n)
 
 
+def effective_split_min_len() -> int:
+    """Rows from which this library splits a decode launch's context (128 unless
+    RETI_RUST_SDPA_2PASS_MIN_LEN is set; the reference's own default is sdpa_2pass_min_len())."""
+    return lib().skv_effective_split_min_len()
+
+
+def kv_bf16_sim_konly() -> bool:
+    """RETI_RUST_KV_BF16_SIM_KONLY (src/decode_resident/utils.rs:245-248)."""
+    return bool(lib().skv_flag_kv_bf16_sim_konly())
+
+
+def kv_bf16_sim_vonly() -> bool:
+    """RETI_RUST_KV_BF16_SIM_VONLY (src/decode_resident/utils.rs:253-256)."""
+    return bool(lib().skv_flag_kv_bf16_sim_vonly())
+
+
+def attention_parallel_threshold() -> int:
+    """RETI_RUST_ATTENTION_PAR_THRESHOLD (src/runtime_flags.rs:641-649)."""
+    return lib().skv_flag_attention_par_threshold()
+
+
+def decode_pipeline_enabled() -> bool:
+    """RETI_RUST_DECODE_PIPELINE (src/runtime_flags.rs:309-313)."""
+    return bool(lib().skv_flag_decode_pipeline())
+
+
 def decode_resident_full_enabled() -> bool:
     return bool(lib().skv_flag_decode_resident_full())
 
@@ -83,6 +109,35 @@ def resident_capacity(prefill_len: int, max_new_tokens: int, draft_headroom: int
     out = ctypes.c_size_t(0)
     ok = lib().skv_resident_capacity(prefill_len, max_new_tokens, draft_headroom, ctypes.byref(out))
     return int(out.value) if ok else None
+
+
+def resident_kv_bytes(capacity: int, kv_dims, elem_bytes: int = 4):
+    """Sum of 2 * capacity * kv_dim * elem_bytes over the layers, or None when a product
+    overflows (check_resident_full_decode_allocation, src/decoder/resident/setup.rs:897-917)."""
+    import ctypes
+    dims = (ctypes.c_size_t * len(kv_dims))(*kv_dims)
+    out = ctypes.c_uint64(0)
+    ok = lib().skv_resident_kv_bytes(capacity, dims, len(kv_dims), elem_bytes, ctypes.byref(out))
+    return int(out.value) if ok else None
+
+
+def memory_projection(current: int, reserved: int, requested: int, limit: int):
+    """(over_limit, projected, available) of MemoryGuard::projection_with_reserved
+    (src/memory_guard.rs:334-362)."""
+    import ctypes
+    proj, avail = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    over = lib().skv_memory_projection(current, reserved, requested, limit, ctypes.byref(proj),
+                                       ctypes.byref(avail))
+    return bool(over), int(proj.value), int(avail.value)
+
+
+def layer_bytes(capacity, q_heads, kv_heads, head_dim, dtype, window=0) -> int:
+    """Device bytes a layer with these arguments takes (skv_layer_bytes)."""
+    import ctypes
+    from ._lib import check
+    out = ctypes.c_uint64(0)
+    check(lib().skv_layer_bytes(capacity, q_heads, kv_heads, head_dim, dtype, window, ctypes.byref(out)))
+    return int(out.value)
 
 
 def f32_to_bf16_bits(value: float) -> int:

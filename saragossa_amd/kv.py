@@ -85,6 +85,15 @@ class DecodeResidentState:
         check(self._l.skv_attn_gate_device(self._h, stream, ctx_ptr, gate_ptr, gate_head_stride,
                                            heads, head_dim, out_ptr))
 
+    def check_allocation(self, requested: int, static_cap: int = 0, headroom: int = 0):
+        """MemoryGuard::check_allocation (src/memory_guard.rs:365-370) against this device:
+        raises MemoryGuardError when the request would pass the ceiling, else returns
+        (available, projected)."""
+        avail, proj = C.c_uint64(0), C.c_uint64(0)
+        check(self._l.skv_check_allocation(self._h, requested, static_cap, headroom, C.byref(avail),
+                                           C.byref(proj)))
+        return int(avail.value), int(proj.value)
+
     def encode_probe_empty_launch(self, stream) -> None:
         """Measurement aid: an empty kernel with the decode launch's shape."""
         check(self._l.skv_probe_empty_launch_device(self._h, stream))

@@ -296,3 +296,73 @@ class HotCache:
             out.append({"session": bytes(s), "hash": bytes(h), "tokens": tok.value,
                         "bytes": nbytes.value})
         return out
+
+
+class WholePromptCache:
+    """The decoder's own whole-prompt prefix cache on the GPU: prefix_cache_get /
+    prefix_cache_put (src/decoder/generation.rs:2998-3025, 3105-3139). ``capacity`` None takes
+    RETI_RUST_PREFIX_CACHE / RETI_RUST_PREFIX_CACHE_CAP (src/runtime_flags.rs:665-678)."""
+
+    def __init__(self, ctx, capacity: Optional[int] = None):
+        self._ctx, self._l = ctx, lib()
+        h = C.c_void_p()
+        if capacity is None:
+            check(self._l.skv_prompt_cache_from_runtime_flags(ctx._h, C.byref(h)))
+        else:
+            check(self._l.skv_prompt_cache_create(ctx._h, capacity, C.byref(h)))
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._l.skv_prompt_cache_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def __len__(self): return self._l.skv_prompt_cache_len(self._h)
+    def capacity(self): return self._l.skv_prompt_cache_capacity(self._h)
+    def estimated_bytes(self): return self._l.skv_prompt_cache_bytes(self._h)
+
+    @property
+    def entries(self) -> List[List[int]]:
+        """Token lists of the entries, most recent first."""
+        out = []
+        for i in range(len(self)):
+            n = C.c_size_t()
+            check(self._l.skv_prompt_cache_entry(self._h, i, C.byref(n), None, 0))
+            buf = np.empty(n.value, dtype=np.uint64)
+            check(self._l.skv_prompt_cache_entry(self._h, i, C.byref(n), buf.ctypes.data_as(C.c_void_p), n.value))
+            out.append([int(t) for t in buf])
+        return out
+
+    def put(self, prompt, layers, state_ptrs=(), state_sizes=(), stream=None) -> None:
+        t = _tok(prompt)
+        pa, sa, n = _ptr_arrays(list(state_ptrs), list(state_sizes))
+        check(self._l.skv_prompt_cache_put(self._h, stream, t.ctypes.data_as(C.c_void_p), t.size,
+                                           _layer_array(layers), len(layers), pa if n else None,
+                                           sa if n else None, n))
+
+    def lookup(self, prompt, layers, state_ptrs=(), state_sizes=(), stream=None) -> int:
+        """The restore half of prefix_cache_get: tokens of the longest cached prefix now in
+        ``layers`` (0 = miss)."""
+        t = _tok(prompt)
+        pa, sa, n = _ptr_arrays(list(state_ptrs), list(state_sizes))
+        cached = C.c_size_t()
+        check(self._l.skv_prompt_cache_get(self._h, stream, t.ctypes.data_as(C.c_void_p), t.size,
+                                           _layer_array(layers), len(layers), pa if n else None,
+                                           sa if n else None, n, C.byref(cached)))
+        return cached.value
+
+    def get(self, prompt, layers, extend: Callable[[int, int], None], state_ptrs=(), state_sizes=(),
+            stream=None) -> Optional[int]:
+        """prefix_cache_get (generation.rs:2998-3025): on a hit the layers hold the whole prompt
+        afterwards (``extend(first, last)`` runs the model over the suffix and appends its rows,
+        then the whole prompt is put) and the cached length is returned; None on a miss."""
+        cached = self.lookup(prompt, layers, state_ptrs, state_sizes, stream)
+        if cached == 0:
+            return None
+        if cached < len(prompt):
+            extend(cached, len(prompt))
+            self.put(prompt, layers, state_ptrs, state_sizes, stream)
+        return cached

@@ -71,7 +71,9 @@ def _flags_in_subprocess(env):
             "full=f.decode_resident_full_enabled(), res=f.decode_resident_enabled(),"
             "serve=f.serve_prefix_cache_enabled(), bt=f.serve_prefix_block_tokens(),"
             "blocks=f.serve_prefix_cache_blocks(), per=f.serve_prefix_blocks_per_session(),"
-            "pc=f.prefix_cache_enabled(), cap=f.prefix_cache_capacity(), chunk=f.prefill_chunk_size())))")
+            "pc=f.prefix_cache_enabled(), cap=f.prefix_cache_capacity(), chunk=f.prefill_chunk_size(),"
+            "split=f.effective_split_min_len(), simk=f.kv_bf16_sim_konly(), simv=f.kv_bf16_sim_vonly(),"
+            "par=f.attention_parallel_threshold(), pipe=f.decode_pipeline_enabled())))")
     full_env = {k: v for k, v in os.environ.items() if not k.startswith("RETI_")}
     full_env.update(env)
     full_env["PYTHONPATH"] = ROOT
@@ -84,7 +86,8 @@ def _flags_in_subprocess(env):
 def test_flag_defaults_match_the_reference():
     d = _flags_in_subprocess({})
     assert d == dict(bf16_s=True, bf16_g=False, flash=True, twopass=True, minlen=2048, full=True,
-                     res=False, serve=True, bt=256, blocks=128, per=128, pc=True, cap=4, chunk=0)
+                     res=False, serve=True, bt=256, blocks=128, per=128, pc=True, cap=4, chunk=0,
+                     split=128, simk=False, simv=False, par=128, pipe=True)
 
 
 def test_flag_overrides_and_precedence():
@@ -96,6 +99,7 @@ def test_flag_overrides_and_precedence():
                               "RETI_RUST_PREFILL_STEP_SIZE": "512", "RETI_SERVE_PREFIX_CACHE": "0"})
     assert (d["bf16_s"], d["bf16_g"]) == (False, False)
     assert (d["flash"], d["twopass"], d["minlen"]) == (False, False, 512)
+    assert d["split"] == 512       # an explicit switch-over length is what the library uses
     assert (d["bt"], d["blocks"], d["per"], d["cap"], d["chunk"], d["serve"]) == (16, 9, 9, 2, 512, False)
     d = _flags_in_subprocess({"RETI_RUST_KV_BF16": "1", "RETI_SERVE_PREFIX_BLOCK_TOKENS": "0",
                               "RETI_SERVE_PREFIX_BLOCKS_PER_SESSION": "3",
@@ -137,3 +141,53 @@ def test_integer_helpers_match_the_oracle():
         assert flags.resident_capacity(a, b, c) == want
     for x in [1.0039062, -0.33325195, 42.125, 0.0, 1e-40, 3.3895314e38]:
         assert flags.f32_to_bf16_bits(x) == int(oracle.f32_to_bf16_bits([x])[0])
+
+
+def test_diagnostic_and_host_loop_flags():
+    # src/decode_resident/utils.rs:245-256; src/runtime_flags.rs:309-313, 641-649
+    d = _flags_in_subprocess({"RETI_RUST_KV_BF16_SIM_KONLY": "1", "RETI_RUST_KV_BF16_SIM_VONLY": "on",
+                              "RETI_RUST_ATTENTION_PAR_THRESHOLD": " 4096 ", "RETI_RUST_DECODE_PIPELINE": "0",
+                              "RETI_RUST_SDPA_2PASS_MIN_LEN": "junk"})
+    assert (d["simk"], d["simv"], d["par"], d["pipe"]) == (True, True, 4096, False)
+    assert d["split"] == 2048 and d["minlen"] == 2048   # set but unparsable: the reference's default
+    d = _flags_in_subprocess({"RETI_RUST_ATTENTION_PAR_THRESHOLD": "-1", "RETI_RUST_DECODE_PIPELINE": "x"})
+    assert (d["par"], d["pipe"]) == (128, True)
+
+
+def test_memory_projection_is_the_reference_guard_arithmetic():
+    # check_allocation_accepts_boundary_and_rejects_overflow (src/memory_guard.rs:748-766):
+    # current 100, cap 150: 50 passes, 51 is refused with available 50 and projected 151
+    assert flags.memory_projection(100, 0, 50, 150) == (False, 150, 50)
+    assert flags.memory_projection(100, 0, 51, 150) == (True, 151, 50)
+    # reservations_are_counted_until_drop (memory_guard.rs:768-786): 100 + 60 reserved, cap 180
+    assert flags.memory_projection(100, 60, 20, 180)[0] is False
+    assert flags.memory_projection(100, 60, 21, 180)[0] is True
+    big = 2 ** 64 - 1
+    assert flags.memory_projection(big, 5, 7, big) == (False, big, 0)      # saturating adds
+    assert flags.memory_projection(10, 0, 1, 5) == (True, 11, 0)           # available floors at 0
+
+
+def test_resident_kv_bytes_and_layer_bytes():
+    # check_resident_full_decode_allocation (src/decoder/resident/setup.rs:897-917): 2 * capacity *
+    # kv_dim * size_of::<f32>() per full-attention layer
+    assert flags.resident_kv_bytes(2304, [1024] * 36) == 36 * 2 * 2304 * 1024 * 4
+    assert flags.resident_kv_bytes(10, []) == 0
+    assert flags.resident_kv_bytes(2 ** 62, [1024]) is None              # "KV résident déborde"
+    # what skv_layer_create takes: whole pages of K and V, table, split partials, staging rows
+    bf = flags.layer_bytes(32768 + 300, 16, 2, 256, skv.DTYPE_BF16)
+    f32 = flags.layer_bytes(32768 + 300, 16, 2, 256, skv.DTYPE_F32)
+    pages = (32768 + 300 + 15) // 16
+    pools = 2 * pages * 2 * 256 * 16 * 2
+    partials = 512 * 16 * (256 + 2) * 4   # the most splits a launch can take
+    assert pools + partials <= bf < pools + partials + 2 ** 16
+    assert 2 * pools + partials <= f32 < 2 * pools + partials + 2 ** 16
+    # a ring layer's size follows its window (plus 32 rows of slack), not its capacity
+    ring = flags.layer_bytes(65536, 16, 8, 256, skv.DTYPE_BF16, 1024)
+    assert 2 * 66 * 8 * 256 * 16 * 2 < ring < 2 * 66 * 8 * 256 * 16 * 2 * 1.2
+    # padded head_dim: 80 -> 128
+    assert flags.layer_bytes(1024, 8, 8, 80, skv.DTYPE_BF16) > 2 * 64 * 8 * 128 * 16 * 2
+    for bad in [(0, 16, 2, 256), (16, 0, 2, 256), (16, 16, 3, 256), (16, 16, 2, 513)]:
+        with pytest.raises(skv.ConfigError):
+            flags.layer_bytes(*bad, skv.DTYPE_BF16)
+    with pytest.raises(skv.ConfigError):
+        flags.layer_bytes(16, 16, 2, 256, 7)

@@ -92,22 +92,22 @@ def test_config4_sliding_window_model_batch1_and_batch4(state):
     gen = torch.Generator(device="cuda").manual_seed(4)
     rng = np.random.default_rng(4)
 
-    def build_sequence(steps):
+    def build_sequence(steps, rows=ctx):
         layers, caches, lays = [], [], []
         for li in range(6):
             is_global = (li + 1) % 6 == 0          # src/decoder.rs:890-898
             w = 0 if is_global else window
-            kv = state.full_attention_bf16(ctx + steps, qh, kvh, hd, window=w)
+            kv = state.full_attention_bf16(rows + steps, qh, kvh, hd, window=w)
             kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
             lay = oracle.layout(qh, kvh, hd, sliding_window=w)
             c = oracle.LayerKvCache("bf16r")
             if is_global:
-                k, v = _seed_device(kv, ctx, kv_dim, gen)
+                k, v = _seed_device(kv, rows, kv_dim, gen)
                 c.append_batch(k, v, lay)
             else:
                 # a local layer only ever attends its last `window` rows, so it starts with its
-                # ring exactly full (position 1024) and wraps from the first decode step on
-                k, v = _seed_device(kv, window, kv_dim, gen)
+                # window exactly full (position 1024) and wraps within the first decode steps
+                k, v = _seed_device(kv, min(window, rows), kv_dim, gen)
                 c.append_batch(k, v, lay)
             layers.append(kv)
             caches.append(c)
@@ -129,11 +129,33 @@ def test_config4_sliding_window_model_batch1_and_batch4(state):
                     worst = max(worst, float(np.abs(o.cpu().numpy() - want).max()))
         return worst
 
+    def run_batched(seqs, steps):
+        """One skv_decode_step_batch_device call per layer covers all the sequences."""
+        worst = 0.0
+        n = len(seqs)
+        for t in range(steps):
+            for li in range(6):
+                q = torch.randn(n, q_dim, device="cuda", generator=gen)
+                k = torch.randn(n, kv_dim, device="cuda", generator=gen)
+                v = torch.randn(n, kv_dim, device="cuda", generator=gen)
+                o = torch.empty(n, q_dim, device="cuda")
+                skv.encode_decode_step_batch([s[0][li] for s in seqs], _stream(),
+                                             [k[i].data_ptr() for i in range(n)],
+                                             [v[i].data_ptr() for i in range(n)],
+                                             [q[i].data_ptr() for i in range(n)],
+                                             [o[i].data_ptr() for i in range(n)])
+                got, qh_, kh_, vh_ = o.cpu().numpy(), q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
+                for i, (_, caches, lays) in enumerate(seqs):
+                    want = oracle.decode_step(caches[li], kh_[i], vh_[i], qh_[i], lays[li])
+                    worst = max(worst, float(np.abs(got[i] - want).max()))
+        return worst
+
+    slack_pages = 2   # a ring keeps 32 rows behind its window
     one = [build_sequence(4)]
     assert run(one, 4) <= 1e-4
-    # ring layers hold exactly their window after wrapping; global layer keeps everything
+    # ring layers hold their window (plus the slack) after wrapping; global layer keeps everything
     layers, caches, _ = one[0]
-    assert layers[0].pages() == window // 16 and layers[5].pages() == (ctx + 4 + 15) // 16
+    assert layers[0].pages() == window // 16 + slack_pages and layers[5].pages() == (ctx + 4 + 15) // 16
     gk, _ = layers[0].read_rows_f32(layers[0].len() - window, window)
     assert np.array_equal(gk, caches[0].keys()[-window:])
     # independent of the oracle: one more attention over the global layer (all 65540 rows) and
@@ -153,12 +175,30 @@ def test_config4_sliding_window_model_batch1_and_batch4(state):
         assert float((o.double() - ref).abs().max()) <= 1e-5, li
     for kv in layers:
         kv.close()
+    del one, layers, caches
+    # batch 4 at full size: four independent sequences at 65536 rows, every layer's step for
+    # the four of them in one launch pair (skv_decode_step_batch_device)
     four = [build_sequence(3) for _ in range(4)]
-    assert run(four, 3) <= 1e-4
+    assert run_batched(four, 3) <= 1e-4
     # sequences are independent: same layer index, different contents
     a, _ = four[0][0][5].read_rows(ctx, 3)
     b, _ = four[1][0][5].read_rows(ctx, 3)
     assert not np.array_equal(a, b)
+    for layers, _, _ in four:
+        for kv in layers:
+            kv.close()
+    del four
+    # sequences of unequal length in one batch: the workgroup budget is shared in proportion,
+    # the short ones take fewer splits (down to one) and their rings are at different fills
+    mixed = [build_sequence(5, rows=r) for r in (65536, 9000, 700, 40)]
+    assert run_batched(mixed, 5) <= 1e-4
+    for (layers, caches, _), r in zip(mixed, (65536, 9000, 700, 40)):
+        gk, gv = layers[5].read_rows_f32(r - 10, 15)
+        assert np.array_equal(gk, caches[5].keys()[r - 10:]) and np.array_equal(gv, caches[5].values()[r - 10:])
+        n = layers[0].len()
+        first = max(0, n - window)
+        gk, _ = layers[0].read_rows_f32(first, n - first)
+        assert np.array_equal(gk, caches[0].keys()[first:])
 
 
 def test_config4_local_layer_chunked_prefill_on_the_ring(state):
@@ -172,7 +212,7 @@ def test_config4_local_layer_chunked_prefill_on_the_ring(state):
     cache = oracle.LayerKvCache("bf16r")
     n_prompt, chunk = 1536 + 100, 512
     kv = state.full_attention_bf16(n_prompt + 8, q_heads, kv_heads, head_dim, window=window)
-    assert kv.pages() == window // 16
+    assert kv.pages() == window // 16 + 2   # the window plus 32 rows of slack
     worst = 0.0
     for first in range(0, n_prompt, chunk):
         c = min(chunk, n_prompt - first)

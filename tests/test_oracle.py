@@ -333,6 +333,20 @@ def test_fused_rms_rope_matches_two_step_and_hand_formula():
         oracle.rms_norm_rope_heads_at(x2, 2, 4, 3, np.ones(4), 0.0, 10000.0, 0)   # odd rope_dims
 
 
+def test_rms_norm_eps_sits_under_the_square_root():
+    # inv_rms = 1 / sqrt(mean_square + eps) (src/decoder/attention_ops.rs:748). With eps = 0.5 the
+    # places it could wrongly sit differ in the first digit: head (3, 4, 0, 0) has mean square
+    # 6.25, so 1/sqrt(6.75) = 0.38490 against 1/(sqrt(6.25) + 0.5) = 0.33333, 1/sqrt(6.25) + 0.5
+    # = 0.9 and 1/sqrt(6.25) = 0.4. Position 0: the rotation is the identity.
+    x = np.array([[3.0, 4.0, 0.0, 0.0, 1.0, -1.0, 1.0, -1.0]], dtype=np.float32)
+    w = np.array([1.0, 2.0, 1.0, 1.0], dtype=np.float32)
+    out = oracle.rms_norm_rope_heads_at(x, 2, 4, 4, w, 0.5, 10000.0, 0)
+    inv0, inv1 = 1.0 / math.sqrt(6.25 + 0.5), 1.0 / math.sqrt(1.0 + 0.5)
+    assert np.allclose(out[0, :4], [3 * inv0, 4 * inv0 * 2, 0, 0], atol=1e-6)
+    assert np.allclose(out[0, 4:], [inv1, -2 * inv1, inv1, -inv1], atol=1e-6)
+    assert abs(out[0, 0] - 3 / (math.sqrt(6.25) + 0.5)) > 0.1   # not eps outside the root
+
+
 # ---- integer policy ----------------------------------------------------------------------
 def test_sdpa_2pass_blocks_and_window_start_and_capacity():
     # src/decode_resident/utils.rs:282-286: 32 blocks at 4096, 64 at 8193, 256 at 32768/33000

@@ -293,3 +293,162 @@ def test_hot_cache_with_recurrent_state_and_skip_when_nothing_to_evict(state):
         hot.remember_prefix_block(root, h1, 64, layers)        # beyond len
     with pytest.raises(skv.ConfigError):
         skv.HotCache(state, 24, 8, 2, layers)                  # not a multiple of the page size
+
+
+def test_config3_full_size_multi_turn_bit_exact_and_reference_lru(state):
+    """BASELINE configs[3] at its full size: 8 sessions share a 4096-token prefix, each adds a
+    256..1024-token history and then a 512-token turn; 16-token hash blocks over the 36 layers
+    of Qwen3-4B KV (8 kv heads, head_dim 128, bf16); the page pool holds 60 % of the distinct
+    blocks, so the LRU evicts. After every turn every row of every layer equals its re-derived
+    value bit for bit, the reused-token count equals the oracle's, and the cache's entries are
+    the oracle's entries in the oracle's recency order (src/serve/state.rs:560-639,
+    src/serve/cache.rs:121-198). Rows are generated and compared on the device."""
+    qh, kvh, hd, nl, bt, n_sessions, vocab = 32, 8, 128, 36, 16, 8, 151936
+    kv_dim = kvh * hd
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(3)
+    shared = rng.integers(0, vocab, size=4096)
+    hist = [rng.integers(0, vocab, size=int(rng.integers(256, 1025))) for _ in range(n_sessions)]
+    turn = [rng.integers(0, vocab, size=512) for _ in range(n_sessions)]
+    base = len(shared) // bt
+    demand = base + sum((len(shared) + len(h) + len(t)) // bt - base for h, t in zip(hist, turn))
+    pool_blocks = int(demand * 0.6)
+
+    def rows_of(layer, tokens, which):
+        t = torch.from_numpy(np.asarray(tokens, dtype=np.int64)).to(dev)
+        c = torch.cumsum(t * 2654435761 % 1000003, 0)
+        pos = torch.arange(t.numel(), device=dev, dtype=torch.int64)
+        d = torch.arange(kv_dim, device=dev, dtype=torch.int64)
+        x = (pos[:, None] * 7919 + c[:, None] * 104729 + d[None, :] * 31 + layer * 1299709 + which * 15485863)
+        x = (x * 6364136223846793005 + 1442695040888963407) >> 40
+        return ((x & 0xffff).to(torch.float32) / 65536.0 - 0.5) * 4.0
+
+    def layers_of(cap, seed):
+        out = []
+        for i in range(nl):
+            kv = state.full_attention_bf16(cap, qh, kvh, hd)
+            kv.set_block_table(np.random.default_rng(seed * 100 + i).permutation(kv.pages()).astype(np.int32))
+            out.append(kv)
+        return out
+
+    proto = layers_of(16, 0)
+    hot = skv.HotCache(state, bt, 10 ** 6, pool_blocks, proto)
+    model = skv.LoadedModelKv(hot, enabled=True)
+    ocache = pc.BlockAwarePrefixCache(bt, 10 ** 6, state_bytes=lambda s, m: 1)
+    over = lambda extra: len(ocache.entries) + extra > pool_blocks
+    odec = SimDecoder()
+    layers = layers_of(len(shared) + 1024 + 512 + 16, 1)
+    gk = torch.empty(5700, kv_dim, device=dev, dtype=torch.int16)
+    gv = torch.empty(5700, kv_dim, device=dev, dtype=torch.int16)
+    totals = dict(reused=0, hits=0)
+
+    def run_turn(tokens):
+        n = len(tokens)
+        for kv in layers:
+            kv.truncate(0)
+        ks = [rows_of(i, tokens, 0) for i in range(nl)]
+        vs = [rows_of(i, tokens, 1) for i in range(nl)]
+
+        def prefill_rows(first, last):
+            for i, kv in enumerate(layers):
+                kv.encode_append_batch(_stream(), ks[i][first].data_ptr(), vs[i][first].data_ptr(), last - first)
+
+        reused = model.prefill_prompt_state([int(t) for t in tokens], None, layers, prefill_rows,
+                                            stream=_stream(), blocks_per_chunk=32)
+        _, want_reused = pc.prefill_prompt_state(ocache, odec, [int(t) for t in tokens], None, over)
+        assert reused == want_reused
+        for i, kv in enumerate(layers):
+            assert kv.len() == n
+            kv.encode_gather(_stream(), 0, n, gk.data_ptr(), gv.data_ptr())
+            assert torch.equal(gk[:n], ks[i].to(torch.bfloat16).view(torch.int16)), f"K of layer {i}"
+            assert torch.equal(gv[:n], vs[i].to(torch.bfloat16).view(torch.int16)), f"V of layer {i}"
+        assert [(e["hash"], e["tokens"]) for e in hot.entries] == [(e.hash, e.tokens) for e in ocache.entries]
+        totals["reused"] += reused
+        totals["hits"] += 1 if reused else 0
+
+    for s in range(n_sessions):
+        run_turn(np.concatenate([shared, hist[s]]))
+    for s in range(n_sessions):
+        run_turn(np.concatenate([shared, hist[s], turn[s]]))
+    assert hot.evictions() > 0 and totals["hits"] >= n_sessions and totals["reused"] > 0
+    assert len(hot) <= pool_blocks
+    hot.close()
+    for kv in proto + layers:
+        kv.close()
+
+
+def test_whole_prompt_cache_follows_the_reference(state, element):
+    """prefix_cache_get / prefix_cache_put (src/decoder/generation.rs:2998-3025, 3105-3139) on
+    the GPU against the oracle's WholePromptCache over the same traffic: same hits, same cached
+    lengths, same entries in the same recency order after every request; after a hit the
+    layers hold the whole prompt's rows bit for bit and the state buffer holds the state that
+    was put with the matched entry."""
+    dims, n_layers = (8, 2, 64), 3
+    kv_dim = dims[1] * dims[2]
+    rng = np.random.default_rng(91)
+    tok = lambda n: [int(t) for t in rng.integers(0, 151936, size=n)]
+    a, b, c, d, e, f = tok(40), tok(30), tok(33), tok(17), tok(50), tok(21)
+    traffic = [a, a + b, c, a[:20], a + b + d, a, e, f, c, a + b + d + tok(3), a + b, []]
+    cache = skv.WholePromptCache(state, capacity=3)
+    ocache = pc.WholePromptCache(capacity=3)
+    assert cache.capacity() == 3 and len(cache) == 0
+    state_of = lambda toks: float(len(toks) * 1000 + sum(toks) % 997)
+    ssm = torch.zeros(300, device="cuda", dtype=torch.float32)
+    ptrs, sizes = [ssm.data_ptr()], [ssm.numel() * 4]
+
+    class S:
+        def __init__(self, n): self.n = n
+        def clone(self): return S(self.n)
+
+    def o_extend(st, toks): st.n += len(toks)
+
+    for step, prompt in enumerate(traffic):
+        layers = make_layers(state, n_layers, 200, dims, seed=step)
+        ssm.fill_(-1.0)
+
+        def extend(first, last):
+            # what the lookup restored is the matched entry's state
+            assert float(ssm[0]) == state_of(prompt[:first]) and float(ssm[-1]) == state_of(prompt[:first])
+            fill(layers, first, last, prompt, kv_dim)
+            ssm.fill_(state_of(prompt))
+
+        got = cache.get(prompt, layers, extend, ptrs, sizes, stream=_stream())
+        want = ocache.get(prompt, o_extend)
+        assert (got is None) == (want is None), step
+        if got is None:
+            if prompt:   # an empty prompt is never cached by the caller (nothing to prefill)
+                fill(layers, 0, len(prompt), prompt, kv_dim)
+                ssm.fill_(state_of(prompt))
+                cache.put(prompt, layers, ptrs, sizes, stream=_stream())
+                ocache.put(prompt, S(len(prompt)))
+        else:
+            assert want.n == len(prompt)
+            torch.cuda.synchronize()
+            check_contents(layers, len(prompt), prompt, kv_dim)
+            assert float(ssm[0]) == state_of(prompt)
+        assert cache.entries == [list(t) for t, _ in ocache.entries], step
+        assert len(cache) <= 3
+        for kv in layers:
+            kv.close()
+    assert cache.estimated_bytes() > 0
+    # the entry a hit restored is independent of what the caller appended afterwards
+    layers = make_layers(state, n_layers, 200, dims, seed=50)
+    top = cache.entries[0]
+    assert cache.lookup(top + [5, 6, 7], layers, ptrs, sizes, stream=_stream()) == len(top)
+    torch.cuda.synchronize()
+    check_contents(layers, len(top), top, kv_dim)
+    # errors precede any copy: too small a layer, a state buffer of another size
+    small = make_layers(state, n_layers, 16, dims, seed=51)
+    with pytest.raises(skv.DimensionError):
+        cache.lookup(top, small, ptrs, sizes, stream=_stream())
+    assert all(kv.len() == 0 for kv in small)
+    with pytest.raises(skv.DimensionError):
+        cache.lookup(top, layers, ptrs, [sizes[0] - 4], stream=_stream())
+    with pytest.raises(skv.DimensionError):
+        cache.put(top[:5], layers, ptrs, sizes)      # the layers hold len(top) rows, not 5
+    # capacity 0: put keeps nothing (generation.rs:3110-3113)
+    off = skv.WholePromptCache(state, capacity=0)
+    off.put(top, layers, ptrs, sizes, stream=_stream())
+    assert len(off) == 0 and off.lookup(top, layers, ptrs, sizes) == 0
+    off.close()
+    cache.close()

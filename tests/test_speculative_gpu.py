@@ -17,7 +17,9 @@ torch = pytest.importorskip("torch")
 @pytest.mark.parametrize("dims,window,base,rounds", [
     ((16, 2, 256), 0, 700, 6),      # full layer, split-K
     ((32, 8, 128), 0, 40, 8),       # short cache
-    ((8, 2, 64), 20, 100, 10),      # ring of 32 rows for a window of 20: 12 rows of slack
+    ((8, 2, 64), 20, 100, 10),      # ring layer, window not a multiple of the page
+    ((8, 2, 64), 64, 200, 10),      # ring layer, window a multiple of 16: the ring's own slack rows
+    ((16, 8, 256), 1024, 1500, 4),  # the local layers of a sliding-window model (window 1024)
 ])
 def test_verify_rows_then_rollback_equals_never_appended(state, dims, window, base, rounds):
     q_heads, kv_heads, head_dim = dims
@@ -54,17 +56,17 @@ def test_verify_rows_then_rollback_equals_never_appended(state, dims, window, ba
     assert np.abs(kv.attention_decode_windowed(q, ws) - oracle.cached_attention_one(q, cache, lay)).max() <= 1e-4
 
 
-def test_rollback_on_a_ring_without_slack_is_an_error_not_stale_data(state):
-    """A ring that holds exactly its window has overwritten the rows a rollback would need:
-    the next attention reports it."""
+def test_rollback_deeper_than_the_rings_slack_is_an_error_not_stale_data(state):
+    """A ring keeps its window plus 32 rows: a rollback of more rows than that needs rows the
+    ring has overwritten, and the next attention reports it instead of reading them."""
     q_heads, kv_heads, head_dim, window = 8, 2, 64, 32
     kv_dim = kv_heads * head_dim
     rng = np.random.default_rng(4)
     kv = state.full_attention_bf16(200, q_heads, kv_heads, head_dim, window=window)
     k = rng.standard_normal((100, kv_dim), dtype=np.float32)
     kv.seed(k, k, 100)
-    q = rng.standard_normal((4, q_heads * head_dim), dtype=np.float32)
-    kv.prefill_rows(q, k[:4], k[:4])
+    q = rng.standard_normal((40, q_heads * head_dim), dtype=np.float32)
+    kv.prefill_rows(q, k[:40], k[:40])
     kv.truncate(101)
     with pytest.raises(skv.DimensionError):
         kv.attention_decode_windowed(q[0], skv.flags.window_start(100, window))
