@@ -225,6 +225,22 @@ int32_t skv_decode_step_device(skv_layer *layer, skv_stream stream, const void *
                                size_t k_off, const void *v_dev, size_t v_off, const float *q_dev,
                                float *out_dev);
 
+/* skv_decode_step_device for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
+ * arguments, same result; the launch's split-K partials live in a static device array of
+ * SKV_STATIC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends,
+ * instead of the layer's own buffers, and the call makes no allocation and frees nothing.
+ * SKV_ERR_DIMENSION when the partials of the launch (q_heads * splits * (head_dim + 2) * 4
+ * bytes; splits follow the context length, 256 workgroups at most) would not fit,
+ * SKV_ERR_CONFIG with RETI_RUST_FLASH_SDPA=0 (the plain kernel allocates its score buffer).
+ * The array keeps the last call's contents and needs no clearing (every partial a launch reads
+ * it has written itself), but all calls on one GPU share it: calls that overlap on one GPU,
+ * on different streams or from different threads, race. */
+#define SKV_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+int32_t skv_decode_step_static_device(skv_layer *layer, skv_stream stream, const void *k_dev,
+                                      size_t k_off, const void *v_dev, size_t v_off,
+                                      const float *q_dev, float *out_dev);
+
 /* Chunked prefill over the cache: appends n_rows rows (k_dev, v_dev: [n_rows, kv_dim] f32)
  * and computes, for every new row i, attention of q_dev[i] over rows 0..len_before+i through
  * the layer's sliding window: cached_attention_prefill_rows

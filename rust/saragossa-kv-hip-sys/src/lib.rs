@@ -28,6 +28,7 @@ pub const SKV_ERR_MEMORY: i32 = 4;
 pub const SKV_DTYPE_F32: i32 = 0;
 pub const SKV_DTYPE_BF16: i32 = 1;
 pub const SKV_PAGE_ROWS: usize = 16;
+pub const SKV_STATIC_SCRATCH_BYTES: usize = 8 << 20;
 
 #[link(name = "saragossa_kv")]
 extern "C" {
@@ -86,6 +87,7 @@ extern "C" {
     pub fn skv_attention_host(layer: *mut skv_layer, q: *const f32, n_elems: usize, window_start: usize, out: *mut f32) -> i32;
     pub fn skv_attention_device(layer: *mut skv_layer, stream: skv_stream, q_dev: *const f32, out_dev: *mut f32, window_start: usize) -> i32;
     pub fn skv_decode_step_device(layer: *mut skv_layer, stream: skv_stream, k_dev: *const c_void, k_off: usize, v_dev: *const c_void, v_off: usize, q_dev: *const f32, out_dev: *mut f32) -> i32;
+    pub fn skv_decode_step_static_device(layer: *mut skv_layer, stream: skv_stream, k_dev: *const c_void, k_off: usize, v_dev: *const c_void, v_off: usize, q_dev: *const f32, out_dev: *mut f32) -> i32;
     pub fn skv_prefill_chunk_device(layer: *mut skv_layer, stream: skv_stream, q_dev: *const f32, k_dev: *const c_void, v_dev: *const c_void, n_rows: usize, out_dev: *mut f32) -> i32;
     pub fn skv_prefill_chunk_host(layer: *mut skv_layer, q: *const f32, k: *const f32, v: *const f32, n_rows: usize, out: *mut f32) -> i32;
     pub fn skv_rope_rotations_host(position: usize, rope_dims: usize, frequency_dim: usize, theta: f32, position_scale: f32, cos_sin_out: *mut f32) -> i32;

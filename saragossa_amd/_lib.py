@@ -65,6 +65,7 @@ SIGNATURES = {
     "skv_layer_bytes": (_i32, [_sz, _sz, _sz, _sz, _i32, _sz, C.POINTER(C.c_uint64)]),
     "skv_check_allocation": (_i32, [_vp, C.c_uint64, C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64),
                                     C.POINTER(C.c_uint64)]),
+    "skv_decode_step_static_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp]),
     "skv_flag_decode_resident_full": (_i32, []),
     "skv_flag_decode_resident": (_i32, []),
     "skv_flag_serve_prefix_cache_enabled": (_i32, []),

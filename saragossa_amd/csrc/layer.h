@@ -14,6 +14,7 @@ using skv::Geom;
 struct skv_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
+    void *static_scratch = nullptr; // this device's copy of the library's static scratch array
     // Split-K partials of multi-query launches (chunked prefill), one buffer per stream the
     // context has seen such a launch on, grown on demand: launches on one stream are ordered by
     // it, launches on different streams never share a buffer. Guarded by arena_mu.

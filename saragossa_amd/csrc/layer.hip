@@ -87,7 +87,34 @@ void ctx_release(skv_ctx *ctx) {
 
 using namespace skv;
 
+// Split-K partials of skv_decode_step_static_device, for callers that cannot allocate. Every
+// GPU the library runs on holds its own copy of the array until the process ends. In host
+// code the array's name is only a stand-in: its device address comes from
+// hipGetSymbolAddress, once per device (static_scratch_ptr), and only that pointer is ever
+// handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[SKV_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[MAX_DEVICES] = {};
+
+// The device address of `scratch` on `device`, which must be the current device.
+hipError_t static_scratch_ptr(int device, void **ptr) {
+    *ptr = nullptr;
+    if (device < 0 || device >= MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = p;
+    }
+    *ptr = g_scratch_ptr[device];
+    return hipSuccess;
+}
 
 int padded_head_dim(size_t hd) {
     for (int p : {32, 64, 128, 256, 512})
@@ -282,13 +309,31 @@ struct PreKv {
     int q_head_stride;  // elements between the heads of q and of gate (0 = head_dim)
 };
 
+// Points the launch's split partials at `buf` instead of the layer's own buffers
+// (decode, one query row): [kv_heads][splits][gqa] of (o[head_dim], m, l).
+int32_t partials_in(void *buf, size_t buf_bytes, DecodeArgs &a) {
+    const Geom &g = a.g;
+    const size_t n_part = (size_t)g.kv_heads * (size_t)a.splits_total * (size_t)g.gqa * (size_t)a.n_queries;
+    const size_t need = n_part * ((size_t)g.head_dim + 2) * sizeof(float);
+    if (need > buf_bytes)
+        return fail(SKV_ERR_DIMENSION, "decode_step_static: partiels split-K de " + std::to_string(need) +
+                                           " o > tampon statique de " + std::to_string(buf_bytes) + " o");
+    a.part_o = reinterpret_cast<float *>(buf);
+    a.part_m = a.part_o + n_part * g.head_dim;
+    a.part_l = a.part_m + n_part;
+    return SKV_OK;
+}
+
 int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float *out_dev,
                          size_t window_start, const float *k_new = nullptr,
                          const float *v_new = nullptr, size_t n_queries = 1,
-                         float attn_scalar = 0.0f, const PreKv *pre = nullptr) {
+                         float attn_scalar = 0.0f, const PreKv *pre = nullptr,
+                         void *static_partials = nullptr) {
     int32_t rc = check_window(L, window_start);
     if (rc) return rc;
     const Geom &g = L->g;
+    if (static_partials && (n_queries != 1 || !uses_flash(L)))
+        return fail(SKV_ERR_CONFIG, "decode_step_static: une ligne de requête, noyau matriciel seulement");
     if (g.f32 && (uses_flash(L) || n_queries > 1)) {
         // the f32 element's matrix kernel (no fused append or pre-KV step): 16 query slots per
         // workgroup, the context split while that leaves compute units idle
@@ -305,6 +350,10 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
                 int32_t rc2 = multi_query_partials(L, s, (size_t)a.splits, n_queries, a);
                 if (rc2) return rc2;
             }
+        }
+        if (static_partials && a.splits > 1) {
+            int32_t rc2 = partials_in(static_partials, SKV_STATIC_SCRATCH_BYTES, a);
+            if (rc2) return rc2;
         }
         SKV_HIP(launch_f32_split(a, s));
         if (a.splits > 1) SKV_HIP(n_queries > 1 ? launch_merge_rows(a, s) : launch_merge(a, s));
@@ -372,6 +421,10 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
             int32_t rc2 = multi_query_partials(L, s, (size_t)a.splits, n_queries, a);
             if (rc2) return rc2;
         }
+    }
+    if (static_partials && a.splits_total > 1) {
+        int32_t rc2 = partials_in(static_partials, SKV_STATIC_SCRATCH_BYTES, a);
+        if (rc2) return rc2;
     }
     if (use_tiles) {
         SKV_HIP(launch_prefill_tiles(a, s));
@@ -448,9 +501,13 @@ int32_t skv_ctx_create(int32_t device, skv_ctx **out) try {
     // orders itself against every blocking stream of the process (a framework's
     // default stream included), so a host call that follows device-side calls on
     // such a stream sees their effect without an explicit wait.
+    // the library's set-up call on this device: the address of the static scratch array here
+    void *static_scratch = nullptr;
+    SKV_HIP(static_scratch_ptr(device, &static_scratch));
     skv_ctx *c = new skv_ctx();
     c->device = device;
     c->stream = nullptr;
+    c->static_scratch = static_scratch;
     c->arena_cap = env_usize("SKV_ARENA_MAX_MB", 4096) << 20;
     *out = c;
     return SKV_OK;
@@ -849,6 +906,48 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
                                   reinterpret_cast<const float *>((const char *)k_dev + k_off),
                                   reinterpret_cast<const float *>((const char *)v_dev + v_off));
     if (rc) L->len -= 1;
+    return rc;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+// skv_decode_step_device with the split partials in the library's static device array
+// instead of the layer's own buffers: nothing here allocates or frees.
+int32_t skv_decode_step_static_device(skv_layer *L, skv_stream stream, const void *k_dev, size_t k_off,
+                                      const void *v_dev, size_t v_off, const float *q_dev,
+                                      float *out_dev) try {
+    if (!L || !k_dev || !v_dev || !q_dev || !out_dev)
+        return fail(SKV_ERR_DEVICE, "decode_step_static: pointeur nul");
+    if (!uses_flash(L))
+        return fail(SKV_ERR_CONFIG, "decode_step_static: le noyau simple (RETI_RUST_FLASH_SDPA=0) alloue son "
+                                    "tampon de scores");
+    void *part = L->ctx->static_scratch;
+    if (!part) return fail(SKV_ERR_DEVICE, "decode_step_static: tampon statique non résolu");
+    if ((k_off | v_off) & 3) return fail(SKV_ERR_DIMENSION, "append device: offset non aligné f32");
+    const float *k = reinterpret_cast<const float *>((const char *)k_dev + k_off);
+    const float *v = reinterpret_cast<const float *>((const char *)v_dev + v_off);
+    hipStream_t s = as_stream(stream);
+    if (!tuning().fused_append || L->g.f32) {
+        // separate launches (the f32 element has no fused append); on a failure after the
+        // append the row stays appended, as with skv_decode_step_device
+        int32_t rc = encode_append(L, s, k, v, 1);
+        if (rc) return rc;
+        return encode_attention(L, s, q_dev, out_dev, skv_window_start(L->len - 1, L->window), nullptr,
+                                nullptr, 1, 0.0f, nullptr, part);
+    }
+    if (L->len >= L->capacity)
+        return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
+                                           std::to_string(L->capacity) + " atteinte (overflow)");
+    const size_t floor_before = L->floor_pos;
+    L->len += 1;
+    if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
+        L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
+    int32_t rc = encode_attention(L, s, q_dev, out_dev, skv_window_start(L->len - 1, L->window), k, v, 1,
+                                  0.0f, nullptr, part);
+    if (rc) {
+        L->len -= 1;
+        L->floor_pos = floor_before;
+    }
     return rc;
 } catch (...) {
     return skv::fail_exception();

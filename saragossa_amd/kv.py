@@ -262,6 +262,12 @@ class FullAttentionState:
         check(self._l.skv_decode_step_device(self._h, stream, k_ptr, k_off, v_ptr, v_off, q_ptr,
                                              out_ptr))
 
+    def encode_decode_step_static(self, stream, k_ptr, k_off, v_ptr, v_off, q_ptr, out_ptr) -> None:
+        """encode_decode_step for callers that cannot allocate: the split partials live in the
+        library's static device array (skv_decode_step_static_device)."""
+        check(self._l.skv_decode_step_static_device(self._h, stream, k_ptr, k_off, v_ptr, v_off,
+                                                    q_ptr, out_ptr))
+
     def encode_decode_step_prekv(self, stream, rope, position, q_ptr, q_off, k_ptr, k_off, v_ptr,
                                  v_off, q_norm_ptr, k_norm_ptr, eps, attn_scalar, out_ptr) -> None:
         """The q/k norms, rotation, query scale, append and attention of

@@ -53,6 +53,7 @@ def test_lib_rs_carries_the_constants_and_handle_types():
     header = open(os.path.join(ROOT, "include", "saragossa_kv.h")).read()
     for name, value in re.findall(r"^#define\s+(SKV_[A-Z0-9_]+)\s+(-?\d+)\b", header, flags=re.M):
         assert re.search(r"pub const %s: \w+ = %s;" % (name, value), text), name
+    assert "pub const SKV_STATIC_SCRATCH_BYTES: usize = 8 << 20;" in text
     for handle in re.findall(r"typedef struct (skv_[a-z_]+) \1;", header):
         assert "pub struct %s " % handle in text, handle
     assert "pub struct skv_hit { pub tokens: usize, pub hash: [u8; 32], pub payload: u64, pub matched_blocks: usize }" in text
