@@ -215,12 +215,12 @@ def bench_prefill(skv, torch, np, state, stream, element="bf16"):
 
 def bench_end_to_end(skv, torch, np, state):
     """BASELINE.json configs[1] end to end: the random-init Qwen3-4B-shaped decoder of the
-    parity test (tests/config1_model.py) with its KV path on the library; 2048-token prompt in
+    parity test (tests/config1_hip.py, which never touches the CPU oracle) with its KV path on the library; 2048-token prompt in
     512-row chunks, then greedy steps. Everything outside the KV path (embedding, projections,
     MLP, norms, lm_head) is plain torch fp32 and only there to drive the KV path at its real
     place in a decoder: the tok/s is dominated by those fp32 matrix products."""
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
-    from config1_model import Config, HipKvPre, Weights, forward
+    from config1_hip import Config, HipKvPre, Weights, forward
     cfg = Config()
     n_prompt, n_new, chunk = 2048, 64, 512
     with torch.no_grad():
@@ -282,6 +282,25 @@ class _TimedHot:
         return self._timed(self.snap_ev, self._hot.remember_prefix_blocks, *a, **kw)
 
 
+def _percentile(values, q):
+    """percentile of bench-serve's summary (src/bench_serve.rs:284-285): nearest rank on the sorted values."""
+    if not values:
+        return 0.0
+    v = sorted(values)
+    return v[min(len(v) - 1, max(0, int(round(q * (len(v) - 1)))))]
+
+
+def config3_traffic(np):
+    """The seeded request stream of BASELINE.json configs[3]: 8 sessions share a 4096-token
+    prefix, each sends prefix + history (256..1024 tokens), then the same plus a 512-token turn."""
+    n_sessions, vocab = 8, 151936
+    rng = np.random.default_rng(3)
+    shared = rng.integers(0, vocab, size=4096)
+    hist = [rng.integers(0, vocab, size=int(rng.integers(256, 1025))) for _ in range(n_sessions)]
+    turn = [rng.integers(0, vocab, size=512) for _ in range(n_sessions)]
+    return shared, hist, turn
+
+
 def bench_config3(args, skv, torch, np, state, stream):
     """BASELINE.json configs[3]: 8 sessions share a 4096-token prefix, each adds a 256..1024
     token history and then a 512-token turn; 16-token hash blocks over 36 layers of Qwen3-4B
@@ -292,10 +311,7 @@ def bench_config3(args, skv, torch, np, state, stream):
     qh, kvh, hd, nl, bt, n_sessions, vocab = 32, 8, 128, 36, 16, 8, 151936
     kv_dim = kvh * hd
     dev = torch.device("cuda:0")
-    rng = np.random.default_rng(3)
-    shared = rng.integers(0, vocab, size=4096)
-    hist = [rng.integers(0, vocab, size=int(rng.integers(256, 1025))) for _ in range(n_sessions)]
-    turn = [rng.integers(0, vocab, size=512) for _ in range(n_sessions)]
+    shared, hist, turn = config3_traffic(np)
     base = len(shared) // bt
     demand = base + sum((len(shared) + len(h) + len(t)) // bt - base for h, t in zip(hist, turn))
     pool_blocks = int(demand * 0.6)
@@ -372,6 +388,16 @@ def bench_config3(args, skv, torch, np, state, stream):
         tot["prompt"] += n
         tot["hits"] += 1 if reused else 0
         tot["turns"] += 1
+        # one line per request, the figures `saragossa serve` returns as x-saragossa-* headers
+        # (ServedCompletion::metric_headers, src/serve/state.rs:59-80) and bench-serve collects
+        # per request (src/bench_serve.rs:249-289), restricted to what the KV side does
+        r_us = sum(e0.elapsed_time(e1) * 1e3 for e0, e1, r in hot.restore_ev if r[0])
+        s_us = sum(e0.elapsed_time(e1) * 1e3 for e0, e1, r in hot.snap_ev)
+        a_us = sum(e0.elapsed_time(e1) * 1e3 for e0, e1, rows in app_ev)
+        requests.append({"index": len(requests), "ok": True, "prompt_tokens": n,
+                         "reused_prefix_tokens": int(reused), "prefill_kv_us": round(r_us + s_us + a_us, 1),
+                         "restore_us": round(r_us, 1), "snapshot_us": round(s_us, 1),
+                         "append_us": round(a_us, 1), "appended_rows": sum(rows for _, _, rows in app_ev)})
         # bit-exact contents after the turn: restored and appended rows alike
         for i, kv in enumerate(layers):
             if kv.len() != n:
@@ -384,6 +410,7 @@ def bench_config3(args, skv, torch, np, state, stream):
                                    "(layer %d, %d reused tokens)" % (i, reused))
         return reused
 
+    requests = []
     t0 = time.perf_counter()
     for s_ in range(n_sessions):
         run_turn(np.concatenate([shared, hist[s_]]), 10 + s_)
@@ -413,6 +440,14 @@ def bench_config3(args, skv, torch, np, state, stream):
         "append": {"rows": tot["appended_rows"], "us": round(tot["append_us"], 1),
                    "us_per_row_all_layers": round(tot["append_us"] / max(tot["appended_rows"], 1), 3)},
         "contents": "bit-exact after every turn (every row of every layer re-derived and compared)",
+        "serve_report": {
+            "summary": {"requested": len(requests), "succeeded": sum(r["ok"] for r in requests),
+                        "failed": sum(not r["ok"] for r in requests), "concurrency": 1,
+                        "prefill_kv_p50_us": round(_percentile([r["prefill_kv_us"] for r in requests], 0.50), 1),
+                        "prefill_kv_p95_us": round(_percentile([r["prefill_kv_us"] for r in requests], 0.95), 1),
+                        "prompt_tokens": tot["prompt"], "reused_prefix_tokens": tot["reused"],
+                        "total_ms": round(wall * 1e3, 1)},
+            "requests": requests},
         "roofline": {"bound": "hbm", "kernel": "page_copy_kernel (restore of the hit blocks, host hash walk included)",
                      "achieved": round(r_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(r_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
@@ -463,7 +498,7 @@ def main() -> int:
                     help="element of the decode leg's caches (f32 is the reference's choice for greedy decoding)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-restore", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--cpu-seconds", type=float, default=3.0)
     ap.add_argument("--end-to-end", action="store_true",
                     help="with --config 1: also run the whole random-init decoder and report tok/s")
     args = ap.parse_args()
@@ -696,6 +731,7 @@ def main() -> int:
                      "restore_traffic_gbps": round(2 * tot_b / tr[len(tr) // 2] / 1e3, 1)}
         del bufs, want
 
+    traffic = MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context and B == 1 and args.element == "bf16" else None
     result = {
         "metric": "KV-path decode us/token @32k ctx (append + paged GQA SDPA, 10 KV layers)"
                   if args.config == 2 else "KV-path decode us/token (append + paged GQA SDPA)",
@@ -724,7 +760,10 @@ def main() -> int:
                                                 "per layer covers the batch, average over the layers)")
                                                % (128 if hd <= 128 else 256),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if not args.context and B == 1 and args.element == "bf16" else None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "traffic_source": None if traffic is None else
+                     "recorded figure, not observed by this run: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over "
+                     "this same command, scaled by a copy of known size (profiles/decode_split_kernel_config2.md)",
                      "bytes_per_launch": launch_bytes,
                      "avg_launch_us": round(kern_avg_us, 2), "median_launch_us": round(kern_med_us, 2),
                      "p10_launch_us": round(kern_ms[len(kern_ms) // 10] * 1e3, 2),

@@ -51,3 +51,45 @@ def test_default_run_prints_one_json_line_with_the_agreed_keys():
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["unit"] == "us/token" and cb["cores"] >= 1 and cb["value"] > 0
     assert d["ceiling"]["read_only_launch_us"] > 0
+
+
+@pytest.mark.gpu
+def test_config3_report_counts_the_reused_tokens_the_reference_algorithm_reuses():
+    """`bench.py --config 3` reports, per request, what `saragossa serve` returns as
+    x-saragossa-prompt-tokens / x-saragossa-reused-prefix-tokens (src/serve/state.rs:59-80) and
+    bench-serve sums up (src/bench_serve.rs:249-289). The reused-token figures must be those of
+    the reference's own prefill_prompt_state over the same request stream with the same pool."""
+    sys.path.insert(0, ROOT)
+    import numpy as np
+
+    import bench
+    from oracle import prefix_cache as pc
+    r = subprocess.run([sys.executable, BENCH, "--config", "3", "--no-cpu-baseline"], capture_output=True,
+                       text=True, timeout=900)
+    assert r.returncode == 0, r.stderr[-2000:]
+    d = json.loads([l for l in r.stdout.splitlines() if l.strip()][-1])
+    rep = d["serve_report"]
+    assert rep["summary"]["requested"] == rep["summary"]["succeeded"] == 16 and rep["summary"]["failed"] == 0
+
+    class Sim(pc.PromptDecoder):
+        class S:
+            def __init__(self, n): self.n = n
+            def clone(self): return Sim.S(self.n)
+        def prefill_uncached(self, tokens): return Sim.S(len(tokens))
+        def extend(self, state, tokens): state.n += len(tokens)
+
+    shared, hist, turn = bench.config3_traffic(np)
+    bt, pool_blocks = 16, d["config"]["pool_blocks"]
+    ocache = pc.BlockAwarePrefixCache(bt, 10 ** 6, state_bytes=lambda s, m: 1)
+    over = lambda extra: len(ocache.entries) + extra > pool_blocks
+    stream = [np.concatenate([shared, h]) for h in hist] + \
+             [np.concatenate([shared, h, t]) for h, t in zip(hist, turn)]
+    want = []
+    for tokens in stream:
+        _, reused = pc.prefill_prompt_state(ocache, Sim(), [int(t) for t in tokens], None, over)
+        want.append((len(tokens), reused))
+    got = [(q["prompt_tokens"], q["reused_prefix_tokens"]) for q in rep["requests"]]
+    assert got == want
+    assert rep["summary"]["reused_prefix_tokens"] == sum(w[1] for w in want) == d["reused_tokens"]
+    assert rep["summary"]["prompt_tokens"] == sum(w[0] for w in want)
+    assert all(q["restore_us"] > 0 for q in rep["requests"] if q["reused_prefix_tokens"])
