@@ -261,8 +261,9 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         if (appends && tid < g.head_dim) k_row = pre_out[rows * PS + tid];
     }
     if (appends) {
-        const int page = a.table[pb_new];
-        const long tile_at = (long)page * g.page_elems + (long)kvh * g.tile_elems;
+        // the page's physical id comes with the arguments: a table lookup here would wait for
+        // every load issued before it, the first K/V page included
+        const long tile_at = (long)a.new_page * g.page_elems + (long)kvh * g.tile_elems;
 #pragma unroll
         for (int u = 0; u < NE; ++u) {
             const int d = tid + u * THREADS;

@@ -258,6 +258,7 @@ void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, si
     a.k_new = k_new;
     a.v_new = v_new;
     a.new_slot = (int)slot_of((long)L->len - 1, g.ring_rows);
+    a.new_page = L->table[(size_t)(a.new_slot >> 4)];
     a.q_vec = (tuning().q_vec && (reinterpret_cast<uintptr_t>(q_dev) & 15) == 0 && (g.head_dim & 7) == 0) ? 1 : 0;
     a.g = g;
 }

@@ -145,6 +145,7 @@ struct DecodeArgs {
     const float *k_new; // [kv_dim] f32
     const float *v_new;
     int new_slot;     // slot that receives the row
+    int new_page;     // physical page of that slot (the host knows its block table)
     // fused pre-KV step (pre != 0): q and the appended k row arrive raw and get the per-head
     // RMSNorm (weights null = none) and the rotation of this position before they are used
     int pre;

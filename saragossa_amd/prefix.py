@@ -184,8 +184,18 @@ class Snapshot:
         self.close()
 
 
+_LAYER_ARRAYS: dict = {}
+
+
 def _layer_array(layers):
-    arr = (C.c_void_p * len(layers))(*[l._h.value for l in layers])
+    """The handles of `layers` as a C array. A server passes the same set of layers at every
+    block boundary, so the last few arrays are kept (keyed by the handles themselves)."""
+    key = tuple(l._h.value for l in layers)
+    arr = _LAYER_ARRAYS.get(key)
+    if arr is None:
+        if len(_LAYER_ARRAYS) >= 16:
+            _LAYER_ARRAYS.clear()
+        arr = _LAYER_ARRAYS[key] = (C.c_void_p * len(key))(*key)
     return arr
 
 
