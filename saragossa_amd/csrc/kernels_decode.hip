@@ -20,6 +20,7 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 constexpr int DEC_MAX_SPLITS = 512;
+constexpr size_t LDS_BYTES = 160 * 1024; // of a gfx950 compute unit
 int decode_max_splits() { return DEC_MAX_SPLITS; }
 
 
@@ -483,9 +484,12 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     // this lane's share of the sum -> the query slot's sum
     l_run = rows_sum(l_run);
 
-    // ---- all wavefronts publish (o, m, l); the workgroup reduces them, four columns per thread
-    __syncthreads(); // the staged queries are no longer needed: the LDS is reused
-    float *xo = reinterpret_cast<float *>(smem);        // [WAVES][rows][OSTRIDE]
+    // ---- all wavefronts publish (o, m, l); the workgroup reduces them, four columns per thread.
+    // Where the LDS holds both, the exchange has an area of its own behind the staged queries,
+    // so a wavefront writes its state as soon as it has finished, without waiting for the
+    // others to stop reading the queries; otherwise the staging area is reused after a barrier.
+    if (a.xchg_off == 0) __syncthreads();
+    float *xo = reinterpret_cast<float *>(reinterpret_cast<char *>(smem) + a.xchg_off); // [WAVES][rows][OSTRIDE]
     float *xm = xo + WAVES * rows * OSTRIDE;            // [WAVES][rows]
     float *xl = xm + WAVES * rows;                      // [WAVES][rows]
     if (n < rows) {
@@ -661,14 +665,18 @@ static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     const int n_slots = a.n_queries * a.g.gqa;
     const int rows = n_slots < 16 ? n_slots : 16;
     const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
-    const size_t lds = stage > xchg ? stage : xchg;
+    const size_t stage16 = (stage + 15) & ~(size_t)15;
+    const bool apart = stage16 + xchg <= LDS_BYTES;
+    const size_t lds = apart ? stage16 + xchg : (stage > xchg ? stage : xchg);
     static std::atomic<uint64_t> lds_ok{0}; // per instantiation
     {
         hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&decode_split_kernel<P, WAVES, MQ, PRE>), lds_ok);
         if (e != hipSuccess) return e;
     }
+    DecodeArgs b = a;
+    b.xchg_off = apart ? (int)stage16 : 0;
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
-    hipLaunchKernelGGL((decode_split_kernel<P, WAVES, MQ, PRE>), grid, dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((decode_split_kernel<P, WAVES, MQ, PRE>), grid, dim3(WAVES * 64), lds, s, b);
     return hipGetLastError();
 }
 
@@ -725,14 +733,18 @@ static hipError_t launch_split_batch(const DecodeBatchArgs &b, int n_seq, int ma
     const size_t stage = (size_t)2 * KK * 64 * sizeof(uint4) + 2 * P * sizeof(uint16_t);
     const int rows = g.gqa < 16 ? g.gqa : 16;
     const size_t xchg = ((size_t)WAVES * rows * (P + 4) + 2 * WAVES * rows) * sizeof(float);
-    const size_t lds = stage > xchg ? stage : xchg;
+    const size_t stage16 = (stage + 15) & ~(size_t)15;
+    const bool apart = stage16 + xchg <= LDS_BYTES;
+    const size_t lds = apart ? stage16 + xchg : (stage > xchg ? stage : xchg);
     static std::atomic<uint64_t> lds_ok{0}; // per instantiation
     {
         hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&decode_split_batch_kernel<P, WAVES>), lds_ok);
         if (e != hipSuccess) return e;
     }
+    DecodeBatchArgs bb = b;
+    for (int i = 0; i < n_seq; ++i) bb.seq[i].xchg_off = apart ? (int)stage16 : 0;
     dim3 grid((unsigned)max_splits, (unsigned)g.kv_heads, (unsigned)n_seq);
-    hipLaunchKernelGGL((decode_split_batch_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, b);
+    hipLaunchKernelGGL((decode_split_batch_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, bb);
     return hipGetLastError();
 }
 

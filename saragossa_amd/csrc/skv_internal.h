@@ -161,6 +161,7 @@ struct DecodeArgs {
     int q_head_stride;
     int q_vec;              // q is 16-byte aligned and head_dim a multiple of 8: 16-byte loads
     int tiles2;             // prefill tile kernel: two 16-slot query tiles per wavefront
+    int xchg_off;           // split kernel: byte offset in LDS of the wavefronts' exchange area (0 = it reuses the staging area); set by the launcher
     Geom g;
 };
 static_assert(sizeof(DecodeArgs) <= 256, "sixteen of them must fit the kernel argument block");
