@@ -212,9 +212,14 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     }
     // Unconditional (a wavefront without pages reads physical page 0 and ignores it): a
     // conditional load here makes the compiler wait for these pages before the queries.
+    // The first page's table entry comes through the scalar unit (the address is the same in
+    // every lane): that read is counted apart from the vector loads above, so the first K/V
+    // request waits for it alone and not for the queries, nor, in the workgroup that
+    // appends, for the new row, which no other workgroup has pulled into a cache.
     uint4 kr[KK], vr[KK];
     {
-        const int pg = page_id(0);
+        typedef const __attribute__((address_space(4))) int32_t *const_i32_ptr;
+        const int pg = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(a.table))[min(pb0 + wave, max(page_hi - 1, 0))];
         load_k<KK>(kr, a, pg, kvh, lane);
         load_v<KK>(vr, a, pg, kvh, lane);
     }
