@@ -10,6 +10,8 @@
 // consecutive contraction steps:
 //   K: float4 unit (m, j, r) = dims 16m + 4j .. +3 of row r, at unit index m * 64 + j * 16 + r
 //   V: float4 unit (c, jj, dd) = rows 4jj .. 4jj+3 of dim 16c + dd, at unit index c * 64 + jj * 16 + dd
+#include <type_traits>
+
 #include "skv_internal.h"
 
 namespace skv {
@@ -144,13 +146,28 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     const float *k_pool = reinterpret_cast<const float *>(a.k_pool);
     const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
     const int last_page = a.page_first + a.n_pages - 1;
+    // Block-table entries of this wavefront's next 64 pages, one per lane, read back with
+    // v_readlane: a page's requests then depend on no load of their own (a table read in
+    // front of every page stalls the wavefront for a round trip before it can ask).
+    int ids = 0;
+    auto fetch_ids = [&](int first_pb) __attribute__((always_inline)) {
+        ids = a.table[min(first_pb + 4 * lane, last_page)];
+    };
+    int ids_base = pb0 + wave; // the page lane 0's entry belongs to
+    fetch_ids(ids_base);
     // (every page of [page_lo, page_hi) is visible to some slot of the tile)
-    auto fetch_tile = [&](int pb, const float *pool, float4_t (&dst)[NT]) {
-        const int page = a.table[min(pb, last_page)];
+    auto fetch_tile = [&](int pb, const float *pool, float4_t (&dst)[NT]) __attribute__((always_inline)) {
+        if (pb >= ids_base + 256) { // uniform: the wavefront has walked 64 pages
+            ids_base += 256;
+            fetch_ids(ids_base);
+        }
+        const int page = __builtin_amdgcn_readlane(ids, (pb - ids_base) >> 2);
         const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
         const float4_t *t = reinterpret_cast<const float4_t *>(pool + tile);
+        // the pages are read once per launch: kept out of the way of the queries, the table
+        // and the partials in the caches
 #pragma unroll
-        for (int m = 0; m < NT; ++m) dst[m] = t[m * 64 + lane];
+        for (int m = 0; m < NT; ++m) dst[m] = __builtin_nontemporal_load(t + m * 64 + lane);
     };
     auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
         fetch_tile(pb, k_pool, kq);
@@ -267,23 +284,123 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
         }
     };
     if constexpr (TWO_PAGES) {
-        // The page after the one being multiplied is already on its way into a second set of
-        // registers: without that every wavefront of the device loads, then multiplies, in
-        // step, and memory idles half the time.
-        auto consume = [&](int at, const float4_t (&kq)[NT], float4_t (&vq)[NT]) {
-            float pv[4];
-            attend(at, kq, pv);
-            mask_v(at, vq);
-            accumulate(vq, pv);
+        // The page after the one being multiplied is on its way into a second set of registers.
+        // A compute unit accepts requests only as fast as memory answers, and a wavefront that
+        // asks for a whole page at once waits at those loads, with its matrix pipe idle (there
+        // is one wavefront per SIMD). The loads of the next page are therefore spread over
+        // the products of this one, one load for every four products (K loads among the QK
+        // products, V loads among the PV products): a load that has to wait holds back only the
+        // few products behind it, which are short of work for the pipe anyway.
+        const int n_it = pb < pb1 ? (pb1 - pb + 3) / 4 : 0;
+        auto next_tile = [&](int at, const float *pool) __attribute__((always_inline)) {
+            const int page = __builtin_amdgcn_readlane(ids, (at - ids_base) >> 2);
+            return reinterpret_cast<const float4_t *>(pool + (((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1)) + lane;
         };
-        while (pb < pb1) {
-            if (pb + 4 < pb1) fetch(pb + 4, k_b, v_b);
-            consume(pb, k_a, v_a);
-            pb += 4;
-            if (pb >= pb1) break;
-            if (pb + 4 < pb1) fetch(pb + 4, k_a, v_a);
-            consume(pb, k_b, v_b);
-            pb += 4;
+        // page `at` from (kq, vq); PREFETCH: page at + 4 into (kn, vn) meanwhile
+        auto step = [&](int at, const float4_t (&kq)[NT], float4_t (&vq)[NT], float4_t (&kn)[NT], float4_t (&vn)[NT],
+                        auto prefetch) __attribute__((always_inline)) {
+            constexpr bool PREFETCH = decltype(prefetch)::value;
+            float pv[4];
+            {
+                const float4_t *kt = PREFETCH ? next_tile(at + 4, k_pool) : nullptr;
+                const int slot_a = at * 16;
+                float4_t s0 = float4_t{0.f, 0.f, 0.f, 0.f}, s1 = float4_t{0.f, 0.f, 0.f, 0.f};
+                if constexpr (PREFETCH) {
+#pragma unroll
+                    for (int m = 0; m < NT; ++m) kn[m] = __builtin_nontemporal_load(kt + m * 64);
+                }
+#pragma unroll
+                for (int m = 0; m < NT; ++m) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][0], qv[m][0], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][1], qv[m][1], s1, 0, 0, 0);
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][2], qv[m][2], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][3], qv[m][3], s1, 0, 0, 0);
+                }
+                if constexpr (PREFETCH) {
+#pragma unroll
+                    for (int m = 0; m < NT; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // one memory read
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0); // four matrix products
+                    }
+                }
+                float sv[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sv[e] = s0[e] + s1[e];
+                const bool interior = g.ring_rows == 0 && slot_a >= t_ws_hi && slot_a + 15 <= t_lim_lo;
+                if (!interior) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int slot = slot_a + j * 4 + e; // this lane's key e
+                        int pos = slot;
+                        if (g.ring_rows > 0) pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+                        sv[e] = (pos >= my_ws && pos <= my_limit) ? sv[e] : -INFINITY;
+                    }
+                }
+                float m_blk = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+                m_blk = rows_max(m_blk);
+                const float m_new = fmaxf(m_run, m_blk);
+                const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+                const float alpha = fast_exp2(m_run - m_safe);
+                float psum = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    pv[e] = fast_exp2(sv[e] - m_safe);
+                    psum += pv[e];
+                }
+                l_run = l_run * alpha + psum;
+                m_run = m_new;
+                if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+                    for (int c = 0; c < NT; ++c) o[c] *= alpha;
+                }
+            }
+            mask_v(at, vq);
+            {
+                const float4_t *vt = PREFETCH ? next_tile(at + 4, v_pool) : nullptr;
+                // contraction step outermost: consecutive products use different accumulators
+                if constexpr (PREFETCH) {
+#pragma unroll
+                    for (int m = 0; m < NT; ++m) vn[m] = __builtin_nontemporal_load(vt + m * 64);
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+#pragma unroll
+                    for (int c = 0; c < NT; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq[c][k], pv[k], o[c], 0, 0, 0);
+                }
+                if constexpr (PREFETCH) {
+#pragma unroll
+                    for (int m = 0; m < NT; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    }
+                }
+            }
+        };
+        const std::true_type with_prefetch{};
+        const std::false_type last_page_of_run{};
+        // The wavefront's pages in runs of up to 64, the block-table entries one register holds:
+        // inside a run no load is conditional (a conditional load makes the compiler wait for
+        // everything in flight where it joins), between runs the pipeline drains once.
+        for (int done = 0; done < n_it;) {
+            const int run = min(n_it - done, 64);
+            const int at0 = pb + 4 * done; // first page of the run, already in (k_a, v_a)
+            int it = 0;
+            for (; it + 2 < run; it += 2) {
+                step(at0 + 4 * it, k_a, v_a, k_b, v_b, with_prefetch);
+                step(at0 + 4 * it + 4, k_b, v_b, k_a, v_a, with_prefetch);
+            }
+            if (run - it == 2) {
+                step(at0 + 4 * it, k_a, v_a, k_b, v_b, with_prefetch);
+                step(at0 + 4 * it + 4, k_b, v_b, k_a, v_a, last_page_of_run);
+            } else {
+                step(at0 + 4 * it, k_a, v_a, k_b, v_b, last_page_of_run);
+            }
+            done += run;
+            if (done < n_it) {
+                ids_base = pb + 4 * done;
+                fetch_ids(ids_base);
+                fetch(ids_base, k_a, v_a);
+            }
         }
     } else {
         // head_dim 257..512: the queries and the accumulators are 256 registers by themselves;
