@@ -169,21 +169,23 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
 #pragma unroll
         for (int m = 0; m < NT; ++m) dst[m] = __builtin_nontemporal_load(t + m * 64 + lane);
     };
-    auto fetch = [&](int pb, float4_t (&kq)[NT], float4_t (&vq)[NT]) {
-        fetch_tile(pb, k_pool, kq);
-        fetch_tile(pb, v_pool, vq);
+    // the page whose table entry lane `idx` of `ids` holds, K then V (no conditional reload)
+    auto fetch = [&](int idx, float4_t (&kq)[NT], float4_t (&vq)[NT]) __attribute__((always_inline)) {
+        const int page = __builtin_amdgcn_readlane(ids, idx);
+        const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
+        const float4_t *kt = reinterpret_cast<const float4_t *>(k_pool + tile) + lane;
+        const float4_t *vt = reinterpret_cast<const float4_t *>(v_pool + tile) + lane;
+#pragma unroll
+        for (int m = 0; m < NT; ++m) kq[m] = __builtin_nontemporal_load(kt + m * 64);
+#pragma unroll
+        for (int m = 0; m < NT; ++m) vq[m] = __builtin_nontemporal_load(vt + m * 64);
     };
     // Up to head_dim 256 a wavefront holds two pages (K and V each); above, one tile at a
-    // time (K, then V in the same registers). The first page is requested before anything
-    // else: the queries' loads ride behind it.
+    // time (K, then V in the same registers).
     constexpr bool TWO_PAGES = P <= 256;
     constexpr int NB = TWO_PAGES ? NT : 1;
     float4_t k_a[NT], v_a[NB], k_b[NB], v_b[NB];
     int pb = pb0 + wave;
-    if (pb < pb1) {
-        if constexpr (TWO_PAGES) fetch(pb, k_a, v_a);
-        else fetch_tile(pb, k_pool, k_a);
-    }
 
     // queries: lane (slot n, group j) holds dims 16m + 4j .. +3 of every block m
     float4_t qv[NT];
@@ -202,6 +204,12 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
                 for (int e = 0; e < 4; ++e) qv[m][e] = qrow[min(m * 16 + j * 4 + e, g.head_dim - 1)];
             }
         }
+        // The first page is requested right behind the queries (loads return in order: in
+        // front of them it would hold them back for the whole page) and without a condition: a
+        // wavefront without pages reads a page it ignores, and the wait for the queries
+        // below counts exactly the page's loads.
+        if constexpr (TWO_PAGES) fetch(0, k_a, v_a);
+        else fetch_tile(min(pb, last_page), k_pool, k_a);
 #pragma unroll
         for (int m = 0; m < NT; ++m) {
 #pragma unroll
@@ -284,13 +292,11 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
         }
     };
     if constexpr (TWO_PAGES) {
-        // The page after the one being multiplied is on its way into a second set of registers.
-        // A compute unit accepts requests only as fast as memory answers, and a wavefront that
-        // asks for a whole page at once waits at those loads, with its matrix pipe idle (there
-        // is one wavefront per SIMD). The loads of the next page are therefore spread over
-        // the products of this one, one load for every four products (K loads among the QK
-        // products, V loads among the PV products): a load that has to wait holds back only the
-        // few products behind it, which are short of work for the pipe anyway.
+        // The page after the one being multiplied is on its way into a second set of registers:
+        // its K tile is asked for in front of this page's QK products, its V tile in front of
+        // the PV products, each tile's loads back to back (spread out among the products, one
+        // load per four, they arrive more slowly: 353.7 against 345.9 us per token at 32768
+        // rows of kv2/hd256).
         const int n_it = pb < pb1 ? (pb1 - pb + 3) / 4 : 0;
         auto next_tile = [&](int at, const float *pool) __attribute__((always_inline)) {
             const int page = __builtin_amdgcn_readlane(ids, (at - ids_base) >> 2);
@@ -315,13 +321,6 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
                     s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][1], qv[m][1], s1, 0, 0, 0);
                     s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][2], qv[m][2], s0, 0, 0, 0);
                     s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][3], qv[m][3], s1, 0, 0, 0);
-                }
-                if constexpr (PREFETCH) {
-#pragma unroll
-                    for (int m = 0; m < NT; ++m) {
-                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // one memory read
-                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0); // four matrix products
-                    }
                 }
                 float sv[4];
 #pragma unroll
@@ -367,13 +366,6 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
 #pragma unroll
                     for (int c = 0; c < NT; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq[c][k], pv[k], o[c], 0, 0, 0);
                 }
-                if constexpr (PREFETCH) {
-#pragma unroll
-                    for (int m = 0; m < NT; ++m) {
-                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-                    }
-                }
             }
         };
         const std::true_type with_prefetch{};
@@ -399,7 +391,7 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
             if (done < n_it) {
                 ids_base = pb + 4 * done;
                 fetch_ids(ids_base);
-                fetch(ids_base, k_a, v_a);
+                fetch(0, k_a, v_a);
             }
         }
     } else {
@@ -470,6 +462,278 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
     }
 }
 
+// ------------------------------------------------------------------------------------
+// The same split launch for one query row (decode) up to head_dim 256, in the shape of the
+// bf16 decode kernel: eight wavefronts, two per SIMD, each with ONE page in its registers
+// (K and V tile, 128 registers at head_dim 256) and the queries in LDS instead of registers.
+// A wavefront that waits for its page, or for the compute unit to accept its next requests,
+// leaves the SIMD's matrix pipe to the other one; with one wavefront per SIMD (the kernel
+// above) the products and the waiting take turns. K registers are refilled right after the
+// QK products that read them, V registers right after the PV products.
+// ------------------------------------------------------------------------------------
+template <int P>
+__global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
+    constexpr int NT = P / 16;
+    constexpr int WAVES = 8;
+    extern __shared__ __attribute__((aligned(16))) float4_t lds8[];
+    float4_t *q_lds = lds8;                  // [NT][64]: lane (slot n, group j) of block m holds dims 16m + 4j .. +3
+    float4_t *xch = lds8 + NT * 64;          // [8 wavefronts][NT][64] o
+    float *xm = reinterpret_cast<float *>(xch + WAVES * NT * 64); // [8][16] m | [8][16] l
+    float *xl = xm + WAVES * 16;
+    const Geom g = a.g;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int j = lane >> 4;
+    const int split = blockIdx.x;
+    const int kvh = blockIdx.y;
+    const int G = g.gqa;
+    const int n_slots = G; // one query row
+    const int slot0 = blockIdx.z * 16;
+    const int my_limit = min(a.q_pos0, a.limit_cap);
+    const int my_ws = a.window > 0 ? max(a.window_start, a.q_pos0 + 1 - a.window) : a.window_start;
+
+    const int page_lo = g.ring_rows > 0 ? 0 : my_ws >> 4;
+    const int page_hi = g.ring_rows > 0 ? a.n_pages : (my_limit >> 4) + 1;
+    const unsigned span = (unsigned)max(page_hi - page_lo, 0);
+    const int pb0 = page_lo + (int)(((unsigned)split * span) / (unsigned)a.splits);
+    const int pb1 = page_lo + (int)(((unsigned)(split + 1) * span) / (unsigned)a.splits);
+    const int pb = pb0 + wave;
+    const int n_it = pb < pb1 ? (pb1 - pb + WAVES - 1) / WAVES : 0;
+
+    const float *k_pool = reinterpret_cast<const float *>(a.k_pool);
+    const float *v_pool = reinterpret_cast<const float *>(a.v_pool);
+    const int last_page = a.page_first + a.n_pages - 1;
+    // block-table entries of this wavefront's next 64 pages, one per lane
+    int ids = 0;
+    auto fetch_ids = [&](int first_pb) __attribute__((always_inline)) {
+        ids = a.table[min(first_pb + WAVES * lane, last_page)];
+    };
+    fetch_ids(pb);
+
+    // ---- queries of the group to LDS, scaled; dims past head_dim are zero
+    {
+        constexpr int QU = (NT * 64 + 511) / 512;
+        float4_t qv[QU];
+#pragma unroll
+        for (int u = 0; u < QU; ++u) {
+            const int idx = min(tid + u * 512, NT * 64 - 1);
+            const int m = idx >> 6, nn = idx & 15, jj = (idx >> 4) & 3;
+            const int slot = min(slot0 + nn, n_slots - 1);
+            const float *qrow = a.q + (long)(kvh * G + slot) * g.head_dim;
+            if (a.q_vec) {
+                qv[u] = *reinterpret_cast<const float4_t *>(qrow + min(m * 16 + jj * 4, g.head_dim - 4));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) qv[u][e] = qrow[min(m * 16 + jj * 4 + e, g.head_dim - 1)];
+            }
+        }
+        // (the first page rides behind the queries: loads return in order)
+        // ---- first page of the wavefront, without a condition (a wavefront without pages reads
+        // a page it ignores): the wait for the queries counts exactly these loads
+        // (placed after the query loads in program order, see below)
+#pragma unroll
+        for (int u = 0; u < QU; ++u) {
+            const int idx = tid + u * 512;
+            if (idx < NT * 64) {
+                const int m = idx >> 6, jj = (idx >> 4) & 3;
+                float4_t v = qv[u];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = m * 16 + jj * 4 + e < g.head_dim ? v[e] * a.qscale : 0.0f;
+                q_lds[idx] = v;
+            }
+        }
+    }
+    float4_t kq[NT], vq[NT];
+    auto tile_of = [&](int idx, const float *pool) __attribute__((always_inline)) {
+        const int page = __builtin_amdgcn_readlane(ids, idx);
+        return reinterpret_cast<const float4_t *>(pool + (((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1)) + lane;
+    };
+    auto load_tile = [&](const float4_t *t, float4_t (&dst)[NT]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int m = 0; m < NT; ++m) dst[m] = __builtin_nontemporal_load(t + m * 64);
+    };
+    load_tile(tile_of(0, k_pool), kq);
+    load_tile(tile_of(0, v_pool), vq);
+    __syncthreads();
+
+    float4_t o[NT];
+#pragma unroll
+    for (int c = 0; c < NT; ++c) o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    auto attend = [&](int at, float (&pv)[4]) __attribute__((always_inline)) {
+        const int slot_a = at * 16;
+        // the queries come from LDS for every page, through an offset the compiler cannot see
+        // through: hoisted out of the page loop they would take 64 registers that do not exist
+        int q_at = lane;
+        asm volatile("" : "+v"(q_at));
+        float4_t s0 = float4_t{0.f, 0.f, 0.f, 0.f}, s1 = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < NT; ++m) {
+            const float4_t qv = q_lds[m * 64 + q_at];
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][0], qv[0], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][1], qv[1], s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][2], qv[2], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[m][3], qv[3], s1, 0, 0, 0);
+        }
+        float sv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sv[e] = s0[e] + s1[e];
+        const bool interior = g.ring_rows == 0 && slot_a >= my_ws && slot_a + 15 <= my_limit;
+        if (!interior) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int slot = slot_a + j * 4 + e;
+                int pos = slot;
+                if (g.ring_rows > 0) pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+                sv[e] = (pos >= my_ws && pos <= my_limit) ? sv[e] : -INFINITY;
+            }
+        }
+        float m_blk = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+        m_blk = rows_max(m_blk);
+        const float m_new = fmaxf(m_run, m_blk);
+        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = fast_exp2(m_run - m_safe);
+        float psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            pv[e] = fast_exp2(sv[e] - m_safe);
+            psum += pv[e];
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) o[c] *= alpha;
+        }
+    };
+    // V of keys that are not attended is replaced by zero on the pages at the edges of the
+    // range (and ring pages): 0 x NaN would be NaN, and the reference never reads those rows
+    // (src/decode_resident/kernels.rs:11-88)
+    auto mask_v = [&](int at) __attribute__((always_inline)) {
+        const int slot_a = at * 16;
+        const bool inside = g.ring_rows == 0 && slot_a >= my_ws && slot_a + 15 <= my_limit;
+        if (inside) return;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int slot = slot_a + j * 4 + k;
+            int pos = slot;
+            if (g.ring_rows > 0) pos = slot <= a.ring_t ? a.ring_base + slot : a.ring_base - g.ring_rows + slot;
+            const bool live = pos >= my_ws && pos <= my_limit;
+#pragma unroll
+            for (int c = 0; c < NT; ++c) vq[c][k] = live ? vq[c][k] : 0.0f;
+        }
+    };
+    auto accumulate = [&](const float (&pv)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+#pragma unroll
+            for (int c = 0; c < NT; ++c) o[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vq[c][k], pv[k], o[c], 0, 0, 0);
+        }
+    };
+    // the wavefront's pages in runs of up to 64 (the table entries one register holds); inside
+    // a run the steady state is unconditional and the last page is peeled, so the waits count
+    // exactly the loads in flight
+    for (int done = 0; done < n_it;) {
+        const int run = min(n_it - done, 64);
+        const int at0 = pb + WAVES * done;
+        for (int it = 0; it + 1 < run; ++it) {
+            const int at = at0 + WAVES * it;
+            float pv[4];
+            attend(at, pv);
+            load_tile(tile_of(it + 1, k_pool), kq);
+            mask_v(at);
+            accumulate(pv);
+            load_tile(tile_of(it + 1, v_pool), vq);
+        }
+        {
+            const int at = at0 + WAVES * (run - 1);
+            float pv[4];
+            attend(at, pv);
+            mask_v(at);
+            accumulate(pv);
+        }
+        done += run;
+        if (done < n_it) {
+            fetch_ids(pb + WAVES * done);
+            load_tile(tile_of(0, k_pool), kq);
+            load_tile(tile_of(0, v_pool), vq);
+        }
+    }
+
+    // ---- the eight wavefronts' states meet in LDS (an area of their own: a wavefront that
+    // has finished does not wait for the others to stop reading the queries)
+    const float l_mine = rows_sum(l_run);
+#pragma unroll
+    for (int c = 0; c < NT; ++c) xch[(wave * NT + c) * 64 + lane] = o[c];
+    if (j == 0) {
+        xm[wave * 16 + n] = m_run;
+        xl[wave * 16 + n] = l_mine;
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    float mw[WAVES];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        mw[w] = xm[w * 16 + n];
+        mx = fmaxf(mx, mw[w]);
+    }
+    const float m_safe = mx == -INFINITY ? 0.0f : mx;
+    float l = 0.0f;
+    float sc[WAVES];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        sc[w] = fast_exp2(mw[w] - m_safe);
+        l += sc[w] * xl[w * 16 + n];
+    }
+    const int slot = slot0 + n;
+    if (slot >= n_slots) return;
+    float *dst;
+    float scale = 1.0f;
+    if (a.splits_total == 1) {
+        scale = 1.0f / l;
+        dst = a.out + (long)(kvh * G + slot) * g.head_dim;
+    } else {
+        const long pidx = ((long)kvh * a.splits_total + a.split_base + split) * n_slots + slot;
+        dst = a.part_o + pidx * g.head_dim;
+        if (j == 0 && wave == 0) {
+            a.part_m[pidx] = mx;
+            a.part_l[pidx] = l;
+        }
+    }
+    // wavefront w finishes the dim tiles c = w, w + 8, ...
+    for (int c = wave; c < NT; c += WAVES) {
+        float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) acc += xch[(w * NT + c) * 64 + lane] * sc[w];
+        acc *= scale;
+        const int col = c * 16 + j * 4;
+        if (a.splits_total > 1 && (g.head_dim & 3) == 0) {
+            if (col < g.head_dim) __builtin_nontemporal_store(acc, reinterpret_cast<float4_t *>(dst + col));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (col + i < g.head_dim) dst[col + i] = acc[i];
+        }
+    }
+}
+
+template <int P>
+static hipError_t launch_f32_decode8(const DecodeArgs &a, dim3 grid, hipStream_t s) {
+    constexpr int NT = P / 16;
+    constexpr size_t lds = (size_t)(NT * 64 + 8 * NT * 64) * sizeof(float4_t) + 2 * 8 * 16 * sizeof(float);
+    static_assert(lds <= 160 * 1024, "queries and the eight wavefronts' states share the LDS of a compute unit");
+    static std::atomic<uint64_t> lds_ok{0}; // per instantiation
+    {
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_decode8_kernel<P>), lds_ok);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((f32_decode8_kernel<P>), grid, dim3(512), lds, s, a);
+    return hipGetLastError();
+}
+
 template <int P>
 static hipError_t launch_f32(const DecodeArgs &a, dim3 grid, hipStream_t s) {
     constexpr size_t lds = (size_t)4 * (P / 16) * 64 * sizeof(float4_t) + 2 * 64 * sizeof(float);
@@ -488,6 +752,15 @@ hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
     if (a.k_new || a.pre) return hipErrorInvalidValue; // no fused append or pre-KV step in this mode
     const int n_slots = a.n_queries * a.g.gqa;
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
+    if (a.n_queries == 1 && a.waves == 8) {
+        switch (a.g.P) {
+        case 32: return launch_f32_decode8<32>(a, grid, s);
+        case 64: return launch_f32_decode8<64>(a, grid, s);
+        case 128: return launch_f32_decode8<128>(a, grid, s);
+        case 256: return launch_f32_decode8<256>(a, grid, s);
+        default: break;
+        }
+    }
     switch (a.g.P) {
     case 32: return launch_f32<32>(a, grid, s);
     case 64: return launch_f32<64>(a, grid, s);
