@@ -22,6 +22,8 @@ namespace {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 } // namespace
 
+bool f32_decode_kernel_serves(const DecodeArgs &a);
+
 // ------------------------------------------------------------------------------------
 // append: rows [n_rows, kv_dim] f32 -> tiles, verbatim. One thread per (row, kv head, four
 // dims): a 16-byte K store and four 4-byte V stores.
@@ -464,22 +466,28 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
 
 // ------------------------------------------------------------------------------------
 // The same split launch for one query row (decode) up to head_dim 256, in the shape of the
-// bf16 decode kernel: eight wavefronts, two per SIMD, each with ONE page in its registers
-// (K and V tile, 128 registers at head_dim 256) and the queries in LDS instead of registers.
-// A wavefront that waits for its page, or for the compute unit to accept its next requests,
-// leaves the SIMD's matrix pipe to the other one; with one wavefront per SIMD (the kernel
+// bf16 decode kernel: eight wavefronts, two per SIMD (four where eight would leave most
+// compute units without a workgroup), each with ONE page in its registers (K and V tile, 128
+// registers at head_dim 256) and the queries in LDS instead of registers. A wavefront that
+// waits for its page, or for the compute unit to accept its next requests, leaves the SIMD's
+// matrix pipe to the other one; with one wavefront per SIMD and two pages each (the kernel
 // above) the products and the waiting take turns. K registers are refilled right after the
 // QK products that read them, V registers right after the PV products.
+// Fused append (k_new non-null): the workgroup whose range holds the new row's page stores
+// the row into the pools for later steps and keeps it in LDS; the wavefront that walks the
+// page patches its registers from there, so nothing is read back in this launch.
 // ------------------------------------------------------------------------------------
-template <int P>
-__global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
+template <int P, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     constexpr int NT = P / 16;
-    constexpr int WAVES = 8;
+    constexpr int THREADS = WAVES * 64;
     extern __shared__ __attribute__((aligned(16))) float4_t lds8[];
     float4_t *q_lds = lds8;                  // [NT][64]: lane (slot n, group j) of block m holds dims 16m + 4j .. +3
-    float4_t *xch = lds8 + NT * 64;          // [8 wavefronts][NT][64] o
-    float *xm = reinterpret_cast<float *>(xch + WAVES * NT * 64); // [8][16] m | [8][16] l
+    float4_t *xch = lds8 + NT * 64;          // [wavefronts][NT][64] o
+    float *xm = reinterpret_cast<float *>(xch + WAVES * NT * 64); // [wavefronts][16] m | l
     float *xl = xm + WAVES * 16;
+    float *new_k = xl + WAVES * 16;          // [P] the appended row
+    float *new_v = new_k + P;
     const Geom g = a.g;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -512,13 +520,32 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
     };
     fetch_ids(pb);
 
+    // ---- fused append: the new row goes to the pools and to LDS
+    const int pb_new = a.new_slot >> 4;
+    const int r_new = a.new_slot & 15;
+    const bool appends = a.k_new != nullptr && pb_new >= pb0 && pb_new < pb1;
+    if (appends) {
+        const long tile_at = ((long)a.new_page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
+        for (int d = tid; d < P; d += THREADS) {
+            float kf = 0.0f, vf = 0.0f;
+            if (d < g.head_dim) {
+                kf = a.k_new[kvh * g.head_dim + d];
+                vf = a.v_new[kvh * g.head_dim + d];
+                const_cast<float *>(k_pool)[tile_at + k_index_f32(r_new, d)] = kf;
+                const_cast<float *>(v_pool)[tile_at + v_index_f32(r_new, d)] = vf;
+            }
+            new_k[d] = kf;
+            new_v[d] = vf;
+        }
+    }
+
     // ---- queries of the group to LDS, scaled; dims past head_dim are zero
     {
-        constexpr int QU = (NT * 64 + 511) / 512;
+        constexpr int QU = (NT * 64 + THREADS - 1) / THREADS;
         float4_t qv[QU];
 #pragma unroll
         for (int u = 0; u < QU; ++u) {
-            const int idx = min(tid + u * 512, NT * 64 - 1);
+            const int idx = min(tid + u * THREADS, NT * 64 - 1);
             const int m = idx >> 6, nn = idx & 15, jj = (idx >> 4) & 3;
             const int slot = min(slot0 + nn, n_slots - 1);
             const float *qrow = a.q + (long)(kvh * G + slot) * g.head_dim;
@@ -529,13 +556,9 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
                 for (int e = 0; e < 4; ++e) qv[u][e] = qrow[min(m * 16 + jj * 4 + e, g.head_dim - 1)];
             }
         }
-        // (the first page rides behind the queries: loads return in order)
-        // ---- first page of the wavefront, without a condition (a wavefront without pages reads
-        // a page it ignores): the wait for the queries counts exactly these loads
-        // (placed after the query loads in program order, see below)
 #pragma unroll
         for (int u = 0; u < QU; ++u) {
-            const int idx = tid + u * 512;
+            const int idx = tid + u * THREADS;
             if (idx < NT * 64) {
                 const int m = idx >> 6, jj = (idx >> 4) & 3;
                 float4_t v = qv[u];
@@ -554,9 +577,13 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
 #pragma unroll
         for (int m = 0; m < NT; ++m) dst[m] = __builtin_nontemporal_load(t + m * 64);
     };
+    // The queries are staged before the first page is asked for: a compute unit accepts
+    // requests only as fast as memory answers them, and a barrier behind a page's loads would
+    // hold every wavefront until the last one's were accepted. The first page comes without a
+    // condition (a wavefront without pages reads a page it ignores).
+    __syncthreads();
     load_tile(tile_of(0, k_pool), kq);
     load_tile(tile_of(0, v_pool), vq);
-    __syncthreads();
 
     float4_t o[NT];
 #pragma unroll
@@ -626,6 +653,26 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
             for (int c = 0; c < NT; ++c) vq[c][k] = live ? vq[c][k] : 0.0f;
         }
     };
+    // the page that receives the appended row takes it from LDS instead of memory
+    auto patch_k = [&](int at) __attribute__((always_inline)) {
+        if (appends && at == pb_new && n == r_new) {
+#pragma unroll
+            for (int m = 0; m < NT; ++m) kq[m] = *reinterpret_cast<const float4_t *>(new_k + m * 16 + j * 4);
+        }
+    };
+    auto patch_v = [&](int at) __attribute__((always_inline)) {
+        if (appends && at == pb_new && j == (r_new >> 2)) {
+            const int e = r_new & 3;
+#pragma unroll
+            for (int c = 0; c < NT; ++c) {
+                const float x = new_v[c * 16 + n];
+                vq[c][0] = e == 0 ? x : vq[c][0];
+                vq[c][1] = e == 1 ? x : vq[c][1];
+                vq[c][2] = e == 2 ? x : vq[c][2];
+                vq[c][3] = e == 3 ? x : vq[c][3];
+            }
+        }
+    };
     auto accumulate = [&](const float (&pv)[4]) __attribute__((always_inline)) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -642,8 +689,10 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
         for (int it = 0; it + 1 < run; ++it) {
             const int at = at0 + WAVES * it;
             float pv[4];
+            patch_k(at);
             attend(at, pv);
             load_tile(tile_of(it + 1, k_pool), kq);
+            patch_v(at);
             mask_v(at);
             accumulate(pv);
             load_tile(tile_of(it + 1, v_pool), vq);
@@ -651,7 +700,9 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
         {
             const int at = at0 + WAVES * (run - 1);
             float pv[4];
+            patch_k(at);
             attend(at, pv);
+            patch_v(at);
             mask_v(at);
             accumulate(pv);
         }
@@ -663,7 +714,7 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
         }
     }
 
-    // ---- the eight wavefronts' states meet in LDS (an area of their own: a wavefront that
+    // ---- the wavefronts' states meet in LDS (an area of their own: a wavefront that
     // has finished does not wait for the others to stop reading the queries)
     const float l_mine = rows_sum(l_run);
 #pragma unroll
@@ -720,17 +771,17 @@ __global__ __launch_bounds__(512) void f32_decode8_kernel(DecodeArgs a) {
     }
 }
 
-template <int P>
-static hipError_t launch_f32_decode8(const DecodeArgs &a, dim3 grid, hipStream_t s) {
+template <int P, int WAVES>
+static hipError_t launch_f32_decode(const DecodeArgs &a, dim3 grid, hipStream_t s) {
     constexpr int NT = P / 16;
-    constexpr size_t lds = (size_t)(NT * 64 + 8 * NT * 64) * sizeof(float4_t) + 2 * 8 * 16 * sizeof(float);
-    static_assert(lds <= 160 * 1024, "queries and the eight wavefronts' states share the LDS of a compute unit");
+    constexpr size_t lds = (size_t)(NT * 64 + WAVES * NT * 64) * sizeof(float4_t) + (2 * WAVES * 16 + 2 * P) * sizeof(float);
+    static_assert(lds <= 160 * 1024, "queries and the wavefronts' states share the LDS of a compute unit");
     static std::atomic<uint64_t> lds_ok{0}; // per instantiation
     {
-        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_decode8_kernel<P>), lds_ok);
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_decode_kernel<P, WAVES>), lds_ok);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((f32_decode8_kernel<P>), grid, dim3(512), lds, s, a);
+    hipLaunchKernelGGL((f32_decode_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
 }
 
@@ -749,18 +800,20 @@ static hipError_t launch_f32(const DecodeArgs &a, dim3 grid, hipStream_t s) {
 // The split launch of an f32 layer; the caller merges (launch_merge for one query row,
 // launch_merge_rows for a chunk) when splits_total > 1.
 hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
-    if (a.k_new || a.pre) return hipErrorInvalidValue; // no fused append or pre-KV step in this mode
+    if (a.pre) return hipErrorInvalidValue; // no fused pre-KV step in this mode
     const int n_slots = a.n_queries * a.g.gqa;
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
-    if (a.n_queries == 1 && a.waves == 8) {
+    if (f32_decode_kernel_serves(a)) {
+        const bool w8 = a.waves == 8;
         switch (a.g.P) {
-        case 32: return launch_f32_decode8<32>(a, grid, s);
-        case 64: return launch_f32_decode8<64>(a, grid, s);
-        case 128: return launch_f32_decode8<128>(a, grid, s);
-        case 256: return launch_f32_decode8<256>(a, grid, s);
+        case 32: return w8 ? launch_f32_decode<32, 8>(a, grid, s) : launch_f32_decode<32, 4>(a, grid, s);
+        case 64: return w8 ? launch_f32_decode<64, 8>(a, grid, s) : launch_f32_decode<64, 4>(a, grid, s);
+        case 128: return w8 ? launch_f32_decode<128, 8>(a, grid, s) : launch_f32_decode<128, 4>(a, grid, s);
+        case 256: return w8 ? launch_f32_decode<256, 8>(a, grid, s) : launch_f32_decode<256, 4>(a, grid, s);
         default: break;
         }
     }
+    if (a.k_new) return hipErrorInvalidValue; // the chunk kernel has no fused append
     switch (a.g.P) {
     case 32: return launch_f32<32>(a, grid, s);
     case 64: return launch_f32<64>(a, grid, s);
@@ -769,6 +822,12 @@ hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
     case 512: return launch_f32<512>(a, grid, s);
     default: return hipErrorInvalidValue;
     }
+}
+
+// One query row of up to 16 heads per group, head_dim up to 256: the decode kernel (which
+// also appends); chunks and wider heads take f32_split_kernel.
+bool f32_decode_kernel_serves(const DecodeArgs &a) {
+    return a.n_queries == 1 && a.g.gqa <= 16 && a.g.P <= 256 && (a.waves == 4 || a.waves == 8);
 }
 
 } // namespace skv

@@ -216,6 +216,10 @@ int32_t check_window(const skv_layer *L, size_t window_start) {
 }
 
 bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L->g.P <= 512; }
+// The attention launch of a decode step can append the row itself: always on bf16 layers,
+// on f32 layers where the f32 decode kernel serves the shape (head_dim up to 256, at most 16
+// heads per group).
+bool fused_append_built(const skv_layer *L) { return !L->g.f32 || (L->g.P <= 256 && L->g.gqa <= 16); }
 // The fused pre-KV step is built up to head_dim 256; wider heads take the separate
 // norm/rotation launches.
 bool wide_heads(const skv_layer *L) { return L->g.P > 256; }
@@ -336,11 +340,14 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     if (static_partials && (n_queries != 1 || !uses_flash(L)))
         return fail(SKV_ERR_CONFIG, "decode_step_static: une ligne de requête, noyau matriciel seulement");
     if (g.f32 && (uses_flash(L) || n_queries > 1)) {
-        // the f32 element's matrix kernel (no fused append or pre-KV step): 16 query slots per
-        // workgroup, the context split while that leaves compute units idle
-        if (k_new || v_new || pre) return fail(SKV_ERR_CONFIG, "KV f32: étape fusionnée non construite");
+        // the f32 element's matrix kernels (no fused pre-KV step): 16 query slots per workgroup,
+        // the context split while that leaves compute units idle; one query row of narrow
+        // heads takes the kernel that can append the row itself
+        if (pre) return fail(SKV_ERR_CONFIG, "KV f32: étape pré-KV fusionnée non construite");
         DecodeArgs a{};
-        fill_decode_args(L, q_dev, out_dev, window_start, nullptr, nullptr, n_queries, decode_target_wgs(), a);
+        fill_decode_args(L, q_dev, out_dev, window_start, k_new, v_new, n_queries, decode_target_wgs(), a);
+        if ((k_new || v_new) && !f32_decode_kernel_serves(a))
+            return fail(SKV_ERR_CONFIG, "KV f32: append fusionné non construit pour cette forme");
         if (attn_scalar > 0.0f) a.qscale = (1.0f / std::sqrt(attn_scalar)) * 1.4426950408889634f;
         if (n_queries > 1) {
             const size_t tiles = (n_queries * (size_t)g.gqa + 15) / 16 * (size_t)g.kv_heads;
@@ -888,7 +895,7 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
     if (!L || !k_dev || !v_dev || !q_dev || !out_dev)
         return fail(SKV_ERR_DEVICE, "decode_step: pointeur nul");
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(L) || L->g.f32) {
+    if (!fused || !uses_flash(L) || !fused_append_built(L)) {
         int32_t rc = skv_append_device(L, stream, k_dev, k_off, v_dev, v_off);
         if (rc) return rc;
         const size_t ws = skv_window_start(L->len - 1, L->window);
@@ -928,8 +935,8 @@ int32_t skv_decode_step_static_device(skv_layer *L, skv_stream stream, const voi
     const float *k = reinterpret_cast<const float *>((const char *)k_dev + k_off);
     const float *v = reinterpret_cast<const float *>((const char *)v_dev + v_off);
     hipStream_t s = as_stream(stream);
-    if (!tuning().fused_append || L->g.f32) {
-        // separate launches (the f32 element has no fused append); on a failure after the
+    if (!tuning().fused_append || !fused_append_built(L)) {
+        // separate launches (wide f32 heads have no fused append); on a failure after the
         // append the row stays appended, as with skv_decode_step_device
         int32_t rc = encode_append(L, s, k, v, 1);
         if (rc) return rc;

@@ -328,6 +328,7 @@ hipError_t launch_gather(const GatherArgs &a, hipStream_t s);
 hipError_t launch_append_f32(const AppendArgs &a, hipStream_t s);
 hipError_t launch_gather_f32(const GatherArgs &a, hipStream_t s);
 hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s);
+bool f32_decode_kernel_serves(const DecodeArgs &a); // the launch takes the kernel that can also append the row
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s);
 hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s);
 hipError_t launch_merge(const DecodeArgs &a, hipStream_t s);        // split-K partials -> context
