@@ -63,6 +63,23 @@ def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> 
     return b
 
 
+def native_remember():
+    """The same 256 one-block remembers from a plain C host (tests/native/kv_c_remember.c, built
+    by __graft_entry__.build()): what the call costs without an interpreter around it. None
+    when the program has not been built."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "native", "kv_c_remember")
+    if not os.path.exists(exe):
+        return None
+    try:
+        run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+        if run.returncode != 0:
+            return {"error": (run.stderr or run.stdout)[-200:]}
+        return json.loads(run.stdout.strip().splitlines()[-1])
+    except Exception as exc:  # a report field, never a reason to lose the bench line
+        return {"error": str(exc)[:200]}
+
+
 def bench_restore(skv, torch, np, state, stream, element="bf16"):
     """Prefix block restore (BASELINE.json configs[3] shapes): the 4096-token shared prefix,
     256 hash blocks of 16 tokens over 36 layers of Qwen3-4B KV (8 kv heads, head_dim 128), is
@@ -170,6 +187,7 @@ def bench_restore(skv, torch, np, state, stream, element="bf16"):
            "frac_of_hbm_peak": round(2 * payload / us / 1e3 / HBM_PEAK_GBPS, 4),
            "snapshot_256_blocks_one_by_one_us": round(snap_us, 1),
            "snapshot_256_blocks_one_by_one_passes_us": [round(t, 1) for t in one_by_one],
+           "snapshot_256_blocks_one_by_one_native": native_remember(),
            "snapshot_256_blocks_one_call_us": round(snap_range_us, 1),
            "snapshot_traffic_gbps": round(2 * payload / snap_range_us / 1e3, 1)}
     for kv in src + dst:

@@ -12,6 +12,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SRC = os.path.join(ROOT, "tests", "native", "kv_c_client.c")
 EXE = os.path.join(ROOT, "tests", "native", "kv_c_client")
+EXE_REMEMBER = os.path.join(ROOT, "tests", "native", "kv_c_remember")
 
 
 def compile_c_client():
@@ -31,7 +32,7 @@ def test_header_is_strict_c11_and_cxx17():
 @pytest.mark.skipif(shutil.which("gcc") is None, reason="gcc not available")
 def test_c_client_compiles_and_links_against_the_library():
     compile_c_client()
-    assert os.path.exists(EXE)
+    assert os.path.exists(EXE) and os.path.exists(EXE_REMEMBER)
 
 
 @pytest.mark.gpu
@@ -41,3 +42,19 @@ def test_c_client_runs_on_the_gpu():
     run = subprocess.run([EXE], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, (run.stdout[-500:], run.stderr[-2000:])
     assert run.stdout.strip().endswith("ok")
+
+
+@pytest.mark.gpu
+def test_c_remember_client_caches_every_block_one_call_per_boundary():
+    """256 block boundaries of a 4096-token prefix over 36 layers, one skv_hot_remember per
+    boundary from plain C: every block is cached, and a call costs a native host a few
+    microseconds (the bound here is loose: it catches a synchronisation or an allocation
+    per call, not a slow machine)."""
+    import json
+    if not os.path.exists(EXE_REMEMBER):
+        compile_c_client()
+    run = subprocess.run([EXE_REMEMBER], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.stdout[-500:], run.stderr[-2000:])
+    rep = json.loads(run.stdout.strip().splitlines()[-1])
+    assert rep["calls"] == 256 and rep["cached"] == 256
+    assert rep["host_us_per_call"] < 40.0, rep
