@@ -220,7 +220,10 @@ int32_t skv_attention_host(skv_layer *layer, const float *q, size_t n_elems, siz
 int32_t skv_attention_device(skv_layer *layer, skv_stream stream, const float *q_dev,
                              float *out_dev, size_t window_start);
 /* append + attention of one token in one call (layers.rs:259-288 does the two
- * encodes back to back). window_start is derived from the layer's window. */
+ * encodes back to back). window_start is derived from the layer's window. On the GPU it is one
+ * launch pair (the attention kernel stores the new row itself) for bf16 layers up to head_dim
+ * 512 and for f32 layers up to head_dim 256 with at most 16 query heads per kv head; other
+ * f32 shapes, and every shape with RETI_RUST_FLASH_SDPA=0, take an append launch first. */
 int32_t skv_decode_step_device(skv_layer *layer, skv_stream stream, const void *k_dev,
                                size_t k_off, const void *v_dev, size_t v_off, const float *q_dev,
                                float *out_dev);
@@ -300,7 +303,9 @@ int32_t skv_rms_norm_rope_decode_host(skv_ctx *ctx, const float *x, const float 
  * sqrt(head_dim / attn_scalar) (encode_query_attention_scale, layers.rs:7-33; an invalid
  * attn_scalar is SKV_ERR_CONFIG), append of (k, v) and attention through the layer's
  * window. q_norm_w / k_norm_w: device f32[head_dim], null = that norm is skipped. The
- * finished q is not written back; the appended k row is the CPU path's row bit for bit. */
+ * finished q is not written back; the appended k row is the CPU path's row bit for bit.
+ * (One launch pair on bf16 layers up to head_dim 256; on f32 layers and wider heads the norm
+ * and rotation, the append and the attention are separate launches with the same result.) */
 int32_t skv_decode_step_prekv_device(skv_layer *layer, skv_stream stream, const skv_rope *rope,
                                      size_t position, const void *q_dev, size_t q_off,
                                      const void *k_dev, size_t k_off, const void *v_dev, size_t v_off,

@@ -1,0 +1,297 @@
+// Measurement aid, not part of the library: what does it cost to merge the split-K partials
+// INSIDE the split launch instead of in a second launch? A kernel shaped like the decode split
+// launch of BASELINE configs[2] (256 workgroups x 512 threads, 256 KiB of K/V streamed and an
+// 8 KiB partial written by each) ends in one of several hand-offs: write-through stores and a
+// counter (one, one per 16 workgroups, one per workgroup), the last workgroup of 128 merging,
+// two levels (16 then 8), a first level among the workgroups of one XCD through its L2 and a
+// second across XCDs; and, for comparison, the plain kernel followed by a second launch.
+// All cross-workgroup data moves with device-scope atomic (write-through, cache-bypassing)
+// accesses ordered by a workgroup barrier, so no L2 write-back or invalidate is needed.
+// Build: make -C saragossa_amd/csrc probes    Run: saragossa_amd/csrc/probes/bin/merge_in_kernel
+#include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+#define CK(x) do{hipError_t e=(x); if(e!=hipSuccess){printf("err %s line %d\n", hipGetErrorString(e), __LINE__); exit(1);} }while(0)
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long u64;
+
+#define AG __HIP_MEMORY_SCOPE_AGENT
+#define WG __HIP_MEMORY_SCOPE_WORKGROUP
+
+__device__ __forceinline__ unsigned xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20); }
+
+template <int SCOPE>
+__device__ __forceinline__ void st4(float *p, float4 v) {
+    u64 a = ((u64)__float_as_uint(v.y) << 32) | __float_as_uint(v.x);
+    u64 b = ((u64)__float_as_uint(v.w) << 32) | __float_as_uint(v.z);
+    __hip_atomic_store((u64 *)p, a, __ATOMIC_RELAXED, SCOPE);
+    __hip_atomic_store((u64 *)p + 1, b, __ATOMIC_RELAXED, SCOPE);
+}
+template <int SCOPE>
+__device__ __forceinline__ float4 ld4(const float *p) {
+    u64 a = __hip_atomic_load((const u64 *)p, __ATOMIC_RELAXED, SCOPE);
+    u64 b = __hip_atomic_load((const u64 *)p + 1, __ATOMIC_RELAXED, SCOPE);
+    return make_float4(__uint_as_float((unsigned)a), __uint_as_float((unsigned)(a >> 32)), __uint_as_float((unsigned)b),
+                       __uint_as_float((unsigned)(b >> 32)));
+}
+
+struct Args {
+    const u32x4 *kpool, *vpool;
+    const int *table;
+    float *part;   // [256][512] float4
+    float *part2;  // [16 or 32][512] float4
+    float *out;    // [2][512] float4
+    unsigned *ctr; // counters, 64 B apart
+    unsigned *xcc_seen; // [256]
+    int n_pages;
+};
+
+template <int MODE>
+__global__ __launch_bounds__(512) void k(Args a) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int split = blockIdx.x, kvh = blockIdx.y, splits = gridDim.x;
+    const int wg = kvh * splits + split;
+    const int pb0 = (int)(((long)split * a.n_pages) / splits), pb1 = (int)(((long)(split + 1) * a.n_pages) / splits);
+    unsigned acc = 0;
+    const size_t page16 = (size_t)2 * 512;
+    for (int pb = pb0 + wave; pb < pb1; pb += 8) {
+        u32x4 kk[8], vv[8];
+        int page = __builtin_amdgcn_readfirstlane(a.table[pb]);
+        const u32x4 *kp = a.kpool + page * page16 + kvh * 512 + lane;
+        const u32x4 *vp = a.vpool + page * page16 + kvh * 512 + lane;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) kk[i] = __builtin_nontemporal_load(kp + i * 64);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vv[i] = __builtin_nontemporal_load(vp + i * 64);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc ^= kk[i].x ^ kk[i].w ^ vv[i].y ^ vv[i].z;
+    }
+    // the workgroup's 8 KiB partial: value wg+1 (+0 from acc, which is a compile-time unknown)
+    const float base = (float)(wg + 1) + (float)(acc == 0x12345678u);
+    float4 pv = make_float4(base, base, base, base);
+    float *mine = a.part + ((size_t)wg * 512 + tid) * 4;
+    __shared__ int last;
+    if (MODE == 0) {
+        { typedef float f4 __attribute__((ext_vector_type(4))); f4 t={pv.x,pv.y,pv.z,pv.w}; __builtin_nontemporal_store(t, (f4 *)mine); }
+        return;
+    }
+    if (MODE == 7 || MODE == 8 || MODE == 9) {
+        *(float4 *)mine = pv; // plain store: reaches this XCD's L2
+    } else {
+        st4<AG>(mine, pv);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (MODE == 1) return;
+    if (MODE == 2 || MODE == 3 || MODE == 4) {
+        if (tid == 0) {
+            unsigned *c = a.ctr + 16 * (MODE == 2 ? 0 : MODE == 3 ? 1 + wg / 16 : 32 + wg);
+            __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, AG);
+        }
+        return;
+    }
+    if (MODE == 5) { // one level, far: 128 arrivals per kv head
+        if (tid == 0) {
+            unsigned t = __hip_atomic_fetch_add(a.ctr + 16 * (300 + kvh), 1u, __ATOMIC_RELAXED, AG);
+            last = ((t + 1) % (unsigned)splits) == 0;
+        }
+        __syncthreads();
+        if (!last) return;
+        float4 s = make_float4(0, 0, 0, 0);
+        for (int i0 = 0; i0 < splits; i0 += 16) {
+            float4 v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = ld4<AG>(a.part + ((size_t)(kvh * splits + i0 + i) * 512 + tid) * 4);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
+        }
+        *(float4 *)(a.out + ((size_t)kvh * 512 + tid) * 4) = s;
+        return;
+    }
+    if (MODE == 6) { // two levels, far: 16 arrivals, then splits/16
+        const int grp = wg / 16;
+        if (tid == 0) {
+            unsigned t = __hip_atomic_fetch_add(a.ctr + 16 * (310 + grp), 1u, __ATOMIC_RELAXED, AG);
+            last = ((t + 1) % 16u) == 0;
+        }
+        __syncthreads();
+        if (!last) return;
+        float4 s = make_float4(0, 0, 0, 0);
+        {
+            float4 v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = ld4<AG>(a.part + ((size_t)(grp * 16 + i) * 512 + tid) * 4);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
+        }
+        st4<AG>(a.part2 + ((size_t)grp * 512 + tid) * 4, s);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        const int n2 = splits / 16;
+        if (tid == 0) {
+            unsigned t = __hip_atomic_fetch_add(a.ctr + 16 * (340 + kvh), 1u, __ATOMIC_RELAXED, AG);
+            last = ((t + 1) % (unsigned)n2) == 0;
+        }
+        __syncthreads();
+        if (!last) return;
+        s = make_float4(0, 0, 0, 0);
+        for (int i = 0; i < n2; ++i) {
+            float4 v = ld4<AG>(a.part2 + ((size_t)(kvh * n2 + i) * 512 + tid) * 4);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        *(float4 *)(a.out + ((size_t)kvh * 512 + tid) * 4) = s;
+        return;
+    }
+    // near modes: group = (kvh, xcc)
+    const unsigned xcc = xcc_id();
+    if (tid == 0) a.xcc_seen[wg] = xcc;
+    if (MODE == 7) { // only the near counter: does an L2-level atomic count all arrivals of this XCD?
+        if (tid == 0) __hip_atomic_fetch_add(a.ctr + 16 * (350 + kvh * 8 + xcc), 1u, __ATOMIC_RELAXED, WG);
+        return;
+    }
+    if (MODE == 9) { // the same counter, all XCDs on ONE address with workgroup scope (expected to lose counts if L2-local)
+        if (tid == 0) __hip_atomic_fetch_add(a.ctr + 16 * 399, 1u, __ATOMIC_RELAXED, WG);
+        return;
+    }
+    if (MODE == 8) {
+        const int per_xcc = splits / 8; // round-robin placement assumed: checked on the host from xcc_seen
+        if (tid == 0) {
+            unsigned t = __hip_atomic_fetch_add(a.ctr + 16 * (370 + kvh * 8 + xcc), 1u, __ATOMIC_RELAXED, WG);
+            last = ((t + 1) % (unsigned)per_xcc) == 0;
+        }
+        __syncthreads();
+        if (!last) return;
+        float4 s = make_float4(0, 0, 0, 0);
+        for (int i0 = 0; i0 < per_xcc; i0 += 16) {
+            float4 v[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int w2 = kvh * splits + (i0 + i) * 8 + (split & 7); // same residue = same XCD under round robin
+                v[i] = ld4<WG>(a.part + ((size_t)w2 * 512 + tid) * 4);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
+        }
+        st4<AG>(a.part2 + ((size_t)(kvh * 8 + (split & 7)) * 512 + tid) * 4, s);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (tid == 0) {
+            unsigned t = __hip_atomic_fetch_add(a.ctr + 16 * (390 + kvh), 1u, __ATOMIC_RELAXED, AG);
+            last = ((t + 1) % 8u) == 0;
+        }
+        __syncthreads();
+        if (!last) return;
+        s = make_float4(0, 0, 0, 0);
+        float4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = ld4<AG>(a.part2 + ((size_t)(kvh * 8 + i) * 512 + tid) * 4);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
+        *(float4 *)(a.out + ((size_t)kvh * 512 + tid) * 4) = s;
+        return;
+    }
+}
+
+__global__ __launch_bounds__(256) void merge_like(const float *part, float *out) {
+    const int t = threadIdx.x, b = blockIdx.x;
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += part[((size_t)(i * 16 + (t >> 4)) * 2048 + b * 16 + (t & 15)) % (256 * 2048)];
+    if ((t >> 4) == 0) out[b * 16 + (t & 15)] = s;
+}
+
+int main() {
+    const int rows = 32768, kv_heads = 2, hd = 256, n_pages = rows / 16, NL = 10, splits = 128;
+    const size_t pool_bytes = (size_t)n_pages * kv_heads * hd * 16 * 2;
+    std::vector<u32x4 *> kp(NL), vp(NL);
+    std::vector<int *> tb(NL);
+    std::mt19937 rng(1);
+    for (int l = 0; l < NL; ++l) {
+        CK(hipMalloc(&kp[l], pool_bytes)); CK(hipMalloc(&vp[l], pool_bytes)); CK(hipMalloc(&tb[l], n_pages * 4));
+        CK(hipMemset(kp[l], 1, pool_bytes)); CK(hipMemset(vp[l], 2, pool_bytes));
+        std::vector<int> t(n_pages);
+        for (int i = 0; i < n_pages; ++i) t[i] = i;
+        std::shuffle(t.begin(), t.end(), rng);
+        CK(hipMemcpy(tb[l], t.data(), n_pages * 4, hipMemcpyHostToDevice));
+    }
+    Args a{};
+    CK(hipMalloc(&a.part, (size_t)256 * 512 * 16)); CK(hipMalloc(&a.part2, (size_t)64 * 512 * 16));
+    CK(hipMalloc(&a.out, 2 * 512 * 16)); CK(hipMalloc(&a.ctr, 64 * 512)); CK(hipMalloc(&a.xcc_seen, 256 * 4));
+    CK(hipMemset(a.ctr, 0, 64 * 512)); CK(hipMemset(a.out, 0, 2 * 512 * 16)); CK(hipMemset(a.xcc_seen, 0xff, 1024));
+    a.n_pages = n_pages;
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    int launches = 0;
+    auto timeit = [&](const char *name, auto launch) {
+        for (int l = 0; l < NL; ++l) launch(l);
+        CK(hipDeviceSynchronize());
+        std::vector<float> ts;
+        for (int r = 0; r < 7; ++r) {
+            const int iters = 10;
+            CK(hipEventRecord(e0));
+            for (int it = 0; it < iters; ++it)
+                for (int l = 0; l < NL; ++l) launch(l);
+            CK(hipEventRecord(e1));
+            CK(hipEventSynchronize(e1));
+            float ms;
+            CK(hipEventElapsedTime(&ms, e0, e1));
+            ts.push_back(ms * 1e3f / (iters * NL));
+        }
+        launches = NL + 7 * 10 * NL;
+        std::sort(ts.begin(), ts.end());
+        printf("%-58s %7.2f us (min %.2f)\n", name, ts[ts.size() / 2], ts[0]);
+        fflush(stdout);
+    };
+    auto check_out = [&](const char *what) {
+        std::vector<float> h(2 * 512 * 4);
+        CK(hipMemcpy(h.data(), a.out, h.size() * 4, hipMemcpyDeviceToHost));
+        // kv head 0: sum of 1..128 = 8256 ; kv head 1: sum of 129..256 = 24640
+        int bad = 0;
+        for (int i = 0; i < 2048; ++i) bad += h[i] != 8256.f;
+        for (int i = 2048; i < 4096; ++i) bad += h[i] != 24640.f;
+        printf("   %s: out[0]=%.0f out[2048]=%.0f mismatches=%d\n", what, h[0], h[2048], bad);
+        CK(hipMemset(a.out, 0, 2 * 512 * 16));
+    };
+#define RUN(M, NAME) timeit(NAME, [&](int l) { Args b = a; b.kpool = kp[l]; b.vpool = vp[l]; b.table = tb[l]; \
+        hipLaunchKernelGGL(k<M>, dim3(splits, kv_heads), dim3(512), 0, 0, b); });
+    RUN(0, "0 nontemporal partial store, end")
+    RUN(1, "1 agent-scope stores + wait + barrier")
+    RUN(2, "2 ... + agent atomic, one counter (256 arrivals)")
+    RUN(3, "3 ... + agent atomic, counter per 16 workgroups")
+    RUN(4, "4 ... + agent atomic, own counter")
+    RUN(5, "5 one level far: last of 128 merges")
+    check_out("mode 5");
+    RUN(6, "6 two levels far: 16 then 8")
+    check_out("mode 6");
+    RUN(7, "7 plain stores + L2-scope atomic per (kvh, xcc)")
+    {
+        std::vector<unsigned> c(16 * 512), x(256);
+        CK(hipMemcpy(c.data(), a.ctr, c.size() * 4, hipMemcpyDeviceToHost));
+        CK(hipMemcpy(x.data(), a.xcc_seen, 1024, hipMemcpyDeviceToHost));
+        printf("   near counters / launches (expect 16 each if counted): ");
+        for (int i = 0; i < 16; ++i) printf("%.2f ", (double)c[16 * (350 + i)] / launches);
+        int rr = 0;
+        for (int w = 0; w < 256; ++w) rr += x[w] == (unsigned)(w % 8);
+        printf("\n   xcc of wg 0..15: ");
+        for (int w = 0; w < 16; ++w) printf("%u ", x[w]);
+        printf("| round-robin matches (last launch): %d of 256\n", rr);
+    }
+    RUN(9, "9 plain stores + L2-scope atomic, ONE address, all XCDs")
+    {
+        std::vector<unsigned> c(16 * 512);
+        CK(hipMemcpy(c.data(), a.ctr, c.size() * 4, hipMemcpyDeviceToHost));
+        printf("   single counter / launches (256 if coherent across XCDs): %.2f\n", (double)c[16 * 399] / launches);
+    }
+    RUN(8, "8 near (16 per XCD, L2) then far (8)")
+    check_out("mode 8");
+    timeit("pair: mode 0 + merge_like launch", [&](int l) {
+        Args b = a; b.kpool = kp[l]; b.vpool = vp[l]; b.table = tb[l];
+        hipLaunchKernelGGL(k<0>, dim3(splits, kv_heads), dim3(512), 0, 0, b);
+        hipLaunchKernelGGL(merge_like, dim3(256), dim3(256), 0, 0, a.part, a.out);
+    });
+    CK(hipDeviceSynchronize());
+    return 0;
+}

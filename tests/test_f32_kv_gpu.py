@@ -177,10 +177,41 @@ def test_snapshot_restore_and_hot_cache_on_f32_layers(state):
 
 
 def test_device_steps_on_f32_layers(state):
-    # the fused entry points run as separate launches on an f32 layer
+    # the pre-KV and gated entry points run as separate launches on an f32 layer
     run_prekv(state, (16, 2, 256), 0, 300, 6, 64, 1.0e7, None, (True, True), element="f32")
     run_prekv(state, (8, 2, 64), 40, 100, 30, 64, 1.0e6, None, (True, False), element="f32")
     run_gated(state, (16, 2, 256), 0, 200, 5, 64, 1.0e7, element="f32")
+
+
+@pytest.mark.parametrize("dims,start,window", [((16, 2, 256), 0, 0), ((16, 2, 256), 4090, 0), ((32, 8, 128), 1000, 0),
+                                               ((8, 2, 64), 15, 0), ((4, 1, 80), 31, 0), ((16, 8, 256), 100, 64),
+                                               ((16, 2, 256), 20000, 0)])
+def test_fused_decode_steps_on_f32_layers(state, dims, start, window):
+    """skv_decode_step_device on an f32 layer is one launch pair: the attention kernel stores the
+    new row itself and patches it into the registers of the wavefront that walks its page
+    (encode_append_kv + attention_decode, src/decode_resident/attention.rs:941-1038). Steps
+    across page boundaries, from an empty cache, on a ring, with four and with eight
+    wavefronts: rows bit for bit, contexts within the f32 bound."""
+    q_dim, kv_dim = dims[0] * dims[2], dims[1] * dims[2]
+    kv, cache, lay, rng = _filled(state, dims, start, seed=start + dims[2], window=window, cap=start + 64)
+    stream = torch.cuda.current_stream().cuda_stream
+    for step in range(35):
+        k = rng.standard_normal(kv_dim, dtype=np.float32)
+        v = rng.standard_normal(kv_dim, dtype=np.float32)
+        q = rng.standard_normal(q_dim, dtype=np.float32)
+        kd, vd, qd = (torch.from_numpy(a).cuda() for a in (k, v, q))
+        out = torch.empty(q_dim, device="cuda")
+        if step % 5 == 4:   # the variant that allocates nothing shares the kernels
+            kv.encode_decode_step_static(stream, kd.data_ptr(), 0, vd.data_ptr(), 0, qd.data_ptr(), out.data_ptr())
+        else:
+            kv.encode_decode_step(stream, kd.data_ptr(), 0, vd.data_ptr(), 0, qd.data_ptr(), out.data_ptr())
+        want = oracle.decode_step(cache, k, v, q, lay)
+        assert np.abs(out.cpu().numpy() - want).max() <= TOL, step
+    n = kv.len()
+    assert n == start + 35
+    keep = min(n, window) if window else n
+    gk, gv = kv.read_rows_f32(n - keep, keep)
+    assert np.array_equal(gk, cache.keys()[n - keep:]) and np.array_equal(gv, cache.values()[n - keep:])
 
 
 def test_decode_step_batch_on_f32_layers(state):
