@@ -166,10 +166,10 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
         const int page = __builtin_amdgcn_readlane(ids, (pb - ids_base) >> 2);
         const long tile = ((long)page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
         const float4_t *t = reinterpret_cast<const float4_t *>(pool + tile);
-        // the pages are read once per launch: kept out of the way of the queries, the table
-        // and the partials in the caches
+        // (plain loads: this kernel serves chunks, whose query tiles share every page through
+        // the L2 of their XCD; the decode kernel below reads its pages once and says so)
 #pragma unroll
-        for (int m = 0; m < NT; ++m) dst[m] = __builtin_nontemporal_load(t + m * 64 + lane);
+        for (int m = 0; m < NT; ++m) dst[m] = t[m * 64 + lane];
     };
     // the page whose table entry lane `idx` of `ids` holds, K then V (no conditional reload)
     auto fetch = [&](int idx, float4_t (&kq)[NT], float4_t (&vq)[NT]) __attribute__((always_inline)) {
@@ -178,9 +178,9 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
         const float4_t *kt = reinterpret_cast<const float4_t *>(k_pool + tile) + lane;
         const float4_t *vt = reinterpret_cast<const float4_t *>(v_pool + tile) + lane;
 #pragma unroll
-        for (int m = 0; m < NT; ++m) kq[m] = __builtin_nontemporal_load(kt + m * 64);
+        for (int m = 0; m < NT; ++m) kq[m] = kt[m * 64];
 #pragma unroll
-        for (int m = 0; m < NT; ++m) vq[m] = __builtin_nontemporal_load(vt + m * 64);
+        for (int m = 0; m < NT; ++m) vq[m] = vt[m * 64];
     };
     // Up to head_dim 256 a wavefront holds two pages (K and V each); above, one tile at a
     // time (K, then V in the same registers).
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
                 float4_t s0 = float4_t{0.f, 0.f, 0.f, 0.f}, s1 = float4_t{0.f, 0.f, 0.f, 0.f};
                 if constexpr (PREFETCH) {
 #pragma unroll
-                    for (int m = 0; m < NT; ++m) kn[m] = __builtin_nontemporal_load(kt + m * 64);
+                    for (int m = 0; m < NT; ++m) kn[m] = kt[m * 64];
                 }
 #pragma unroll
                 for (int m = 0; m < NT; ++m) {
@@ -361,7 +361,7 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
                 // contraction step outermost: consecutive products use different accumulators
                 if constexpr (PREFETCH) {
 #pragma unroll
-                    for (int m = 0; m < NT; ++m) vn[m] = __builtin_nontemporal_load(vt + m * 64);
+                    for (int m = 0; m < NT; ++m) vn[m] = vt[m * 64];
                 }
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
