@@ -477,7 +477,7 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
 // the row into the pools for later steps and keeps it in LDS; the wavefront that walks the
 // page patches its registers from there, so nothing is read back in this launch.
 // ------------------------------------------------------------------------------------
-template <int P, int WAVES>
+template <int P, int WAVES, bool PRE>
 __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     constexpr int NT = P / 16;
     constexpr int THREADS = WAVES * 64;
@@ -498,6 +498,7 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     const int kvh = blockIdx.y;
     const int G = g.gqa;
     const int n_slots = G; // one query row
+    const int q_stride = a.q_head_stride > 0 ? a.q_head_stride : g.head_dim;
     const int slot0 = blockIdx.z * 16;
     const int my_limit = min(a.q_pos0, a.limit_cap);
     const int my_ws = a.window > 0 ? max(a.window_start, a.q_pos0 + 1 - a.window) : a.window_start;
@@ -524,12 +525,69 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     const int pb_new = a.new_slot >> 4;
     const int r_new = a.new_slot & 15;
     const bool appends = a.k_new != nullptr && pb_new >= pb0 && pb_new < pb1;
+
+    // ---- PRE: q and the new k row arrive raw; the per-head RMSNorm and the rotation of the
+    // position are applied here, in LDS (the area the wavefronts' states use at the end), with
+    // the arithmetic and the order of rms_norm_rope_heads_at (src/decoder/attention_ops.rs:682-777),
+    // so that the finished rows, and the k row this launch stores, equal the CPU path's.
+    constexpr int PS = P + 1;      // row stride: lanes walking different rows hit different banks
+    constexpr int SQS = P + 4;     // squares: 16-byte aligned rows
+    constexpr int PRE_ROWS = 17;   // 16 query slots + the k row
+    float *pre_raw = reinterpret_cast<float *>(xch);   // [PRE_ROWS][PS]
+    float *pre_out = pre_raw + PRE_ROWS * PS;          // [PRE_ROWS][PS]
+    float *pre_wq = pre_out + PRE_ROWS * PS;           // [P]
+    float *pre_wk = pre_wq + P;                        // [P]
+    float *pre_rope = pre_wk + P;                      // [P]: (cos, sin) pairs
+    float *pre_inv = pre_rope + P;                     // [PRE_ROWS] (+5 keeps pre_sq 16-byte aligned)
+    float *pre_sq = pre_inv + PRE_ROWS + 5;            // [PRE_ROWS][SQS]
+    static_assert(!PRE || ((size_t)(2 * PRE_ROWS * PS + 3 * P + PRE_ROWS + 5 + PRE_ROWS * SQS) * sizeof(float) <=
+                           (size_t)WAVES * NT * 64 * sizeof(float4_t)),
+                  "the pre-KV scratch fits the exchange area it borrows");
+    const int rows = min(16, n_slots - slot0);
+    if constexpr (PRE) {
+        auto sq_of = [](float x) {
+#pragma clang fp contract(off)
+            return x * x;
+        };
+        for (int e = tid; e < rows * P; e += THREADS) {
+            const int r = e / P, c = e % P;
+            const float x = c < g.head_dim ? a.q[(long)(kvh * G + slot0 + r) * q_stride + c] : 0.0f;
+            pre_raw[r * PS + c] = x;
+            pre_sq[r * SQS + c] = sq_of(x);
+        }
+        for (int c = tid; c < P; c += THREADS) {
+            const float x = (appends && c < g.head_dim) ? a.k_new[kvh * g.head_dim + c] : 0.0f;
+            pre_raw[rows * PS + c] = x;
+            pre_sq[rows * SQS + c] = sq_of(x);
+            pre_wq[c] = (a.q_norm_w && c < g.head_dim) ? a.q_norm_w[c] : 1.0f;
+            pre_wk[c] = (a.k_norm_w && c < g.head_dim) ? a.k_norm_w[c] : 1.0f;
+            pre_rope[c] = (a.rope && c < a.rope_dims) ? a.rope[c] : 0.0f;
+        }
+        __syncthreads();
+        const int n_rows = rows + (appends ? 1 : 0);
+        if (tid < n_rows) {
+            const bool is_k = tid == rows;
+            const bool has_norm = is_k ? a.k_norm_w != nullptr : a.q_norm_w != nullptr;
+            pre_inv[tid] = has_norm ? head_inv_rms_sq(pre_sq + tid * SQS, P, g.head_dim, a.eps) : 1.0f;
+        }
+        __syncthreads();
+        const float *rope = a.rope ? pre_rope : nullptr;
+        for (int e = tid; e < n_rows * P; e += THREADS) {
+            const int r = e / P, c = e % P;
+            if (c < g.head_dim) {
+                const bool is_k = r == rows;
+                const float *w = is_k ? (a.k_norm_w ? pre_wk : nullptr) : (a.q_norm_w ? pre_wq : nullptr);
+                pre_out[r * PS + c] = norm_rope_elem(pre_raw + r * PS, c, pre_inv[r], w, rope, a.rope_dims, a.rope_style);
+            }
+        }
+        __syncthreads();
+    }
     if (appends) {
         const long tile_at = ((long)a.new_page * g.page_elems + (long)kvh * g.tile_elems) >> 1;
         for (int d = tid; d < P; d += THREADS) {
             float kf = 0.0f, vf = 0.0f;
             if (d < g.head_dim) {
-                kf = a.k_new[kvh * g.head_dim + d];
+                kf = PRE ? pre_out[rows * PS + d] : a.k_new[kvh * g.head_dim + d];
                 vf = a.v_new[kvh * g.head_dim + d];
                 const_cast<float *>(k_pool)[tile_at + k_index_f32(r_new, d)] = kf;
                 const_cast<float *>(v_pool)[tile_at + v_index_f32(r_new, d)] = vf;
@@ -548,12 +606,18 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
             const int idx = min(tid + u * THREADS, NT * 64 - 1);
             const int m = idx >> 6, nn = idx & 15, jj = (idx >> 4) & 3;
             const int slot = min(slot0 + nn, n_slots - 1);
-            const float *qrow = a.q + (long)(kvh * G + slot) * g.head_dim;
-            if (a.q_vec) {
-                qv[u] = *reinterpret_cast<const float4_t *>(qrow + min(m * 16 + jj * 4, g.head_dim - 4));
-            } else {
+            if constexpr (PRE) {
+                const float *qrow = pre_out + (slot - slot0) * PS;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) qv[u][e] = qrow[min(m * 16 + jj * 4 + e, g.head_dim - 1)];
+            } else {
+                const float *qrow = a.q + (long)(kvh * G + slot) * q_stride;
+                if (a.q_vec) {
+                    qv[u] = *reinterpret_cast<const float4_t *>(qrow + min(m * 16 + jj * 4, g.head_dim - 4));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) qv[u][e] = qrow[min(m * 16 + jj * 4 + e, g.head_dim - 1)];
+                }
             }
         }
 #pragma unroll
@@ -743,9 +807,11 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     if (slot >= n_slots) return;
     float *dst;
     float scale = 1.0f;
+    const float *gp = nullptr;
     if (a.splits_total == 1) {
         scale = 1.0f / l;
         dst = a.out + (long)(kvh * G + slot) * g.head_dim;
+        if (a.gate) gp = a.gate + (long)(kvh * G + slot) * q_stride;
     } else {
         const long pidx = ((long)kvh * a.splits_total + a.split_base + split) * n_slots + slot;
         dst = a.part_o + pidx * g.head_dim;
@@ -761,6 +827,11 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
         for (int w = 0; w < WAVES; ++w) acc += xch[(w * NT + c) * 64 + lane] * sc[w];
         acc *= scale;
         const int col = c * 16 + j * 4;
+        if (gp) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (col + i < g.head_dim) acc[i] *= sigmoid_gate(gp[col + i]);
+        }
         if (a.splits_total > 1 && (g.head_dim & 3) == 0) {
             if (col < g.head_dim) __builtin_nontemporal_store(acc, reinterpret_cast<float4_t *>(dst + col));
         } else {
@@ -771,18 +842,22 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     }
 }
 
-template <int P, int WAVES>
-static hipError_t launch_f32_decode(const DecodeArgs &a, dim3 grid, hipStream_t s) {
+template <int P, int WAVES, bool PRE>
+static hipError_t launch_f32_decode_pre(const DecodeArgs &a, dim3 grid, hipStream_t s) {
     constexpr int NT = P / 16;
     constexpr size_t lds = (size_t)(NT * 64 + WAVES * NT * 64) * sizeof(float4_t) + (2 * WAVES * 16 + 2 * P) * sizeof(float);
     static_assert(lds <= 160 * 1024, "queries and the wavefronts' states share the LDS of a compute unit");
     static std::atomic<uint64_t> lds_ok{0}; // per instantiation
     {
-        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_decode_kernel<P, WAVES>), lds_ok);
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_decode_kernel<P, WAVES, PRE>), lds_ok);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((f32_decode_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, a);
+    hipLaunchKernelGGL((f32_decode_kernel<P, WAVES, PRE>), grid, dim3(WAVES * 64), lds, s, a);
     return hipGetLastError();
+}
+template <int P, int WAVES>
+static hipError_t launch_f32_decode(const DecodeArgs &a, dim3 grid, hipStream_t s) {
+    return a.pre ? launch_f32_decode_pre<P, WAVES, true>(a, grid, s) : launch_f32_decode_pre<P, WAVES, false>(a, grid, s);
 }
 
 template <int P>
@@ -800,7 +875,6 @@ static hipError_t launch_f32(const DecodeArgs &a, dim3 grid, hipStream_t s) {
 // The split launch of an f32 layer; the caller merges (launch_merge for one query row,
 // launch_merge_rows for a chunk) when splits_total > 1.
 hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
-    if (a.pre) return hipErrorInvalidValue; // no fused pre-KV step in this mode
     const int n_slots = a.n_queries * a.g.gqa;
     dim3 grid((unsigned)a.splits, (unsigned)a.g.kv_heads, (unsigned)((n_slots + 15) / 16));
     if (f32_decode_kernel_serves(a)) {
@@ -813,7 +887,7 @@ hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
         default: break;
         }
     }
-    if (a.k_new) return hipErrorInvalidValue; // the chunk kernel has no fused append
+    if (a.k_new || a.pre) return hipErrorInvalidValue; // the chunk kernel has no fused append or pre-KV step
     switch (a.g.P) {
     case 32: return launch_f32<32>(a, grid, s);
     case 64: return launch_f32<64>(a, grid, s);

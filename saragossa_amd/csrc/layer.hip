@@ -340,14 +340,24 @@ int32_t encode_attention(skv_layer *L, hipStream_t s, const float *q_dev, float 
     if (static_partials && (n_queries != 1 || !uses_flash(L)))
         return fail(SKV_ERR_CONFIG, "decode_step_static: une ligne de requête, noyau matriciel seulement");
     if (g.f32 && (uses_flash(L) || n_queries > 1)) {
-        // the f32 element's matrix kernels (no fused pre-KV step): 16 query slots per workgroup,
-        // the context split while that leaves compute units idle; one query row of narrow
-        // heads takes the kernel that can append the row itself
-        if (pre) return fail(SKV_ERR_CONFIG, "KV f32: étape pré-KV fusionnée non construite");
+        // the f32 element's matrix kernels: 16 query slots per workgroup, the context split while
+        // that leaves compute units idle; one query row of narrow heads takes the kernel that
+        // can append the row (and norm and rotate q and k) itself
         DecodeArgs a{};
         fill_decode_args(L, q_dev, out_dev, window_start, k_new, v_new, n_queries, decode_target_wgs(), a);
-        if ((k_new || v_new) && !f32_decode_kernel_serves(a))
-            return fail(SKV_ERR_CONFIG, "KV f32: append fusionné non construit pour cette forme");
+        if ((k_new || v_new || pre) && !f32_decode_kernel_serves(a))
+            return fail(SKV_ERR_CONFIG, "KV f32: étape fusionnée non construite pour cette forme");
+        if (pre) {
+            a.pre = 1;
+            a.rope = pre->rope;
+            a.q_norm_w = pre->q_norm_w;
+            a.k_norm_w = pre->k_norm_w;
+            a.eps = pre->eps;
+            a.rope_dims = pre->rope ? pre->rope_dims : 0;
+            a.rope_style = pre->rope_style;
+            a.gate = pre->gate;
+            a.q_head_stride = pre->q_head_stride;
+        }
         if (attn_scalar > 0.0f) a.qscale = (1.0f / std::sqrt(attn_scalar)) * 1.4426950408889634f;
         if (n_queries > 1) {
             const size_t tiles = (n_queries * (size_t)g.gqa + 15) / 16 * (size_t)g.kv_heads;
@@ -1292,7 +1302,7 @@ static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope,
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     hipStream_t s = as_stream(stream);
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(L) || wide_heads(L) || L->g.gqa > 16 || L->g.f32) {
+    if (!fused || !uses_flash(L) || wide_heads(L) || L->g.gqa > 16) {
         // the same step as separate launches: norm + rotation of q and k, append, attention, gate
         NormRopeArgs n{};
         n.x = q;

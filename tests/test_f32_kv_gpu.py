@@ -177,7 +177,7 @@ def test_snapshot_restore_and_hot_cache_on_f32_layers(state):
 
 
 def test_device_steps_on_f32_layers(state):
-    # the pre-KV and gated entry points run as separate launches on an f32 layer
+    # the pre-KV and gated entry points are one launch pair on an f32 layer too (head_dim <= 256)
     run_prekv(state, (16, 2, 256), 0, 300, 6, 64, 1.0e7, None, (True, True), element="f32")
     run_prekv(state, (8, 2, 64), 40, 100, 30, 64, 1.0e6, None, (True, False), element="f32")
     run_gated(state, (16, 2, 256), 0, 200, 5, 64, 1.0e7, element="f32")
