@@ -1,0 +1,365 @@
+// Measurement aid, not part of the library: how fast do the matrix pipes of the whole device
+// run the instruction streams of the prefill kernel when nothing else is in the way? Every
+// variant issues the matrix products of a 512-row chunk over 32768 cached rows at head_dim 256
+// (two bf16 terms per operand: 550 GFLOP issued); variants 0 to 3 without page copies, softmax or
+// barriers:
+//   0  32x32x16 products, operands in registers, one wavefront per SIMD
+//   1  the same with the A operands read from LDS (16-byte K reads, two 8-byte V reads)
+//   2  16x16x32 products, operands in registers, one wavefront per SIMD
+//   3  16x16x32 products as the prefill kernel issues them: eight wavefronts (two per SIMD), one
+//      16-slot query tile each, K and V operands of a page pair read from LDS as 16-byte units
+//   4-7  variant 3 plus the other parts of the prefill kernel's step: online softmax (4), and the
+//      barrier of every step (5); barrier and page copies through registers into LDS without
+//      the softmax (6); all of them (7)
+// Each variant runs twice: on a constant bit pattern and on random values in (-0.25, 0.25). The
+// clock the device sustains under the matrix pipes depends on how many operand bits toggle, so
+// the second figure is the one a kernel on real data can be held against.
+// Build: make -C saragossa_amd/csrc probes    Run: saragossa_amd/csrc/probes/bin/mfma_stream
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float float16_t;
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+#define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e_)); exit(1);} } while (0)
+
+constexpr int LDS_BYTES = 65536; // two page pairs: [K tile A | K tile B | V tile A | V tile B] of 8 KiB each
+
+template <int T>
+__global__ __launch_bounds__(T == 3 ? 512 : 256) void stream(const uint4 *src, float *out, int n_pairs) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < LDS_BYTES / 16; i += blockDim.x) reinterpret_cast<uint4 *>(lds)[i] = src[i];
+    __syncthreads();
+    float acc = 0.f;
+    if (T == 3) {
+        bf16x8_t qh[8], ql[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            qh[s] = __builtin_bit_cast(bf16x8_t, src[(s * 64 + lane) & 4095]);
+            ql[s] = __builtin_bit_cast(bf16x8_t, src[(s * 64 + lane + 512) & 4095]);
+        }
+        float4_t o[16];
+#pragma unroll
+        for (int c = 0; c < 16; ++c) o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int it = 0; it < n_pairs; ++it) {
+            const uint4 *kt_a = reinterpret_cast<const uint4 *>(lds + (it & 1) * 32768);
+            const uint4 *kt_b = kt_a + 512;
+            const uint4 *vt = kt_a + 1024;
+            float4_t sa0 = {0.f, 0.f, 0.f, 0.f}, sa1 = sa0, sb0 = sa0, sb1 = sa0;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const bf16x8_t ka = __builtin_bit_cast(bf16x8_t, kt_a[kk * 64 + lane]);
+                const bf16x8_t kb = __builtin_bit_cast(bf16x8_t, kt_b[kk * 64 + lane]);
+                sa0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qh[kk], sa0, 0, 0, 0);
+                sa1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, ql[kk], sa1, 0, 0, 0);
+                sb0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qh[kk], sb0, 0, 0, 0);
+                sb1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, ql[kk], sb1, 0, 0, 0);
+            }
+            // stand-ins for the probabilities: any bf16 operands that depend on the scores
+            const float4_t sx = sa0 + sa1, sy = sb0 + sb1;
+            const bf16x8_t ph = __builtin_bit_cast(bf16x8_t, make_uint4(__float_as_uint(sx[0]), __float_as_uint(sx[1]),
+                                                                        __float_as_uint(sy[0]), __float_as_uint(sy[1])));
+            const bf16x8_t pl = __builtin_bit_cast(bf16x8_t, make_uint4(__float_as_uint(sx[2]), __float_as_uint(sx[3]),
+                                                                        __float_as_uint(sy[2]), __float_as_uint(sy[3])));
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const bf16x8_t v0 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + lane]);
+                const bf16x8_t v1 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + 64 + lane]);
+                o[2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, ph, o[2 * kk], 0, 0, 0);
+                o[2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, ph, o[2 * kk + 1], 0, 0, 0);
+                o[2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, pl, o[2 * kk], 0, 0, 0);
+                o[2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, pl, o[2 * kk + 1], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) acc += o[c][0] + o[c][1] + o[c][2] + o[c][3];
+    } else {
+        const int h = lane >> 5, c = lane & 31;
+        bf16x8_t q[32];
+#pragma unroll
+        for (int s = 0; s < 32; ++s) q[s] = __builtin_bit_cast(bf16x8_t, src[(s * 64 + lane) & 4095]);
+        float16_t o[8], s0, s1;
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[b][r] = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            s0[r] = 0.f;
+            s1[r] = 0.f;
+        }
+        for (int it = 0; it < n_pairs; ++it) {
+            const char *buf = lds + (it & 1) * 32768;
+            if (T == 2) {
+                float4_t a4[8];
+#pragma unroll
+                for (int b = 0; b < 8; ++b) a4[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < 128; ++s)
+                    a4[s & 7] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(q[s & 31], q[(s + 1) & 31], a4[s & 7], 0, 0, 0);
+#pragma unroll
+                for (int b = 0; b < 8; ++b)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[b][r] += a4[b][r];
+                continue;
+            }
+            // K operand of step s: key = lane % 32 (page A or B by bit 4), dims 16s + 8h .. + 7
+            const char *kbase = buf + (c >> 4) * 8192 + (h * 16 + (c & 15)) * 16;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                bf16x8_t ka = q[(s + 16) & 31];
+                if (T == 1) ka = *reinterpret_cast<const bf16x8_t *>(kbase + s * 512);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, q[2 * s], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, q[2 * s + 1], s1, 0, 0, 0);
+            }
+            // V operand of (dim block b, page t): dim = 32b + lane % 32, two groups of four keys
+            const char *vbase = buf + 16384 + (h * 16 + (c & 15)) * 16 + (c >> 4) * 8;
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    bf16x8_t va = q[(b * 2 + t + 7) & 31];
+                    if (T == 1) {
+                        const uint2 x0 = *reinterpret_cast<const uint2 *>(vbase + t * 8192 + b * 1024);
+                        const uint2 x1 = *reinterpret_cast<const uint2 *>(vbase + t * 8192 + b * 1024 + 512);
+                        va = __builtin_bit_cast(bf16x8_t, make_uint4(x0.x, x0.y, x1.x, x1.y));
+                    }
+                    o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, q[t], o[b], 0, 0, 0);
+                    o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, q[t + 2], o[b], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc += o[b][r];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc += s0[r] + s1[r];
+    }
+    out[blockIdx.x * blockDim.x + tid] = acc;
+}
+
+constexpr int PG = 4;
+constexpr int TILE_U4 = 512;
+constexpr int BUF_U4 = PG * 2 * TILE_U4;
+constexpr int STEP_LDS_BYTES = 2 * BUF_U4 * 16; // two buffers of four pages: 128 KiB
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float rows_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+// The prefill kernel's step on top of variant 3. F bit 0: the online softmax between the two
+// groups of products; bit 1: the workgroup barrier of every step (four pages); bit 2: the page
+// copies of the next step (memory -> registers -> LDS, V tiles interleaved in 8-byte halves)
+template <int F>
+__global__ __launch_bounds__(512) void skel(const uint4 *pool, const int *table, float *out, int n_steps) {
+    extern __shared__ __attribute__((aligned(16))) uint4 kv_lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    for (int i = tid; i < STEP_LDS_BYTES / 16; i += 512) kv_lds[i] = pool[i];
+    __syncthreads();
+    bf16x8_t qh[8], ql[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        qh[s] = __builtin_bit_cast(bf16x8_t, pool[(s * 64 + lane) & 4095]);
+        ql[s] = __builtin_bit_cast(bf16x8_t, pool[(s * 64 + lane + 512) & 4095]);
+    }
+    float4_t o[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) o[c] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    uint4 stage[PG][2];
+    auto fetch = [&](int step) {
+#pragma unroll
+        for (int pg = 0; pg < PG; ++pg) {
+            const int page = table[(blockIdx.x * 7 + step * PG + pg) & 2047];
+            const uint4 *kp = pool + (long)page * 2048;     // [K kvh0 | K kvh1 | V kvh0 | V kvh1]-like spacing
+            const uint4 *vp = kp + 1024;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = tid + u * 512;
+                stage[pg][u] = i < TILE_U4 ? kp[i] : vp[i - TILE_U4];
+            }
+        }
+    };
+    auto store = [&](uint4 *buf) {
+#pragma unroll
+        for (int pg = 0; pg < PG; ++pg) {
+            uint4 *pair = buf + (pg >> 1) * 4 * TILE_U4;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int i = tid + u * 512;
+                const uint4 x = stage[pg][u];
+                if (i < TILE_U4) pair[(pg & 1) * TILE_U4 + i] = x;
+                else {
+                    const int iv = i - TILE_U4;
+                    uint2 *dst = reinterpret_cast<uint2 *>(pair + 2 * TILE_U4 + (iv >> 6) * 128 + (iv & 63)) + (pg & 1);
+                    dst[0] = make_uint2(x.x, x.y);
+                    dst[128] = make_uint2(x.z, x.w);
+                }
+            }
+        }
+    };
+    for (int step = 0; step < n_steps; ++step) {
+        if (F & 4) fetch(step + 1);
+#pragma unroll
+        for (int pp = 0; pp < PG / 2; ++pp) {
+            const uint4 *kt_a = kv_lds + (step & 1) * BUF_U4 + pp * 4 * TILE_U4;
+            const uint4 *kt_b = kt_a + TILE_U4;
+            const uint4 *vt = kt_a + 2 * TILE_U4;
+            float4_t sa0 = {0.f, 0.f, 0.f, 0.f}, sa1 = sa0, sb0 = sa0, sb1 = sa0;
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const bf16x8_t ka = __builtin_bit_cast(bf16x8_t, kt_a[kk * 64 + lane]);
+                const bf16x8_t kb = __builtin_bit_cast(bf16x8_t, kt_b[kk * 64 + lane]);
+                sa0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qh[kk], sa0, 0, 0, 0);
+                sa1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, ql[kk], sa1, 0, 0, 0);
+                sb0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qh[kk], sb0, 0, 0, 0);
+                sb1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, ql[kk], sb1, 0, 0, 0);
+            }
+            bf16x8_t ph, pl;
+            const float4_t xa = sa0 + sa1, xb = sb0 + sb1;
+            if (F & 1) {
+                float sv[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { sv[i] = xa[i]; sv[4 + i] = xb[i]; }
+                float m_blk = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+                m_blk = rows_max(m_blk);
+                const float m_new = fmaxf(m_run, m_blk);
+                const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+                const float alpha = fast_exp2(m_run - m_safe);
+                float psum = 0.0f;
+                uint32_t pb_[8], rb_[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float pv = fast_exp2(sv[e] - m_safe);
+                    psum += pv;
+                    pb_[e] = __float_as_uint(pv);
+                    rb_[e] = __float_as_uint(pv - __uint_as_float(pb_[e] & 0xffff0000u));
+                }
+                ph = __builtin_bit_cast(bf16x8_t, make_uint4(__builtin_amdgcn_perm(pb_[1], pb_[0], 0x07060302u), __builtin_amdgcn_perm(pb_[3], pb_[2], 0x07060302u),
+                                                             __builtin_amdgcn_perm(pb_[5], pb_[4], 0x07060302u), __builtin_amdgcn_perm(pb_[7], pb_[6], 0x07060302u)));
+                pl = __builtin_bit_cast(bf16x8_t, make_uint4(__builtin_amdgcn_perm(rb_[1], rb_[0], 0x07060302u), __builtin_amdgcn_perm(rb_[3], rb_[2], 0x07060302u),
+                                                             __builtin_amdgcn_perm(rb_[5], rb_[4], 0x07060302u), __builtin_amdgcn_perm(rb_[7], rb_[6], 0x07060302u)));
+                l_run = l_run * alpha + psum;
+                m_run = m_new;
+                if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+#pragma unroll
+                    for (int c = 0; c < 16; ++c) o[c] *= alpha;
+                }
+            } else {
+                ph = __builtin_bit_cast(bf16x8_t, make_uint4(__float_as_uint(xa[0]), __float_as_uint(xa[1]), __float_as_uint(xb[0]), __float_as_uint(xb[1])));
+                pl = __builtin_bit_cast(bf16x8_t, make_uint4(__float_as_uint(xa[2]), __float_as_uint(xa[3]), __float_as_uint(xb[2]), __float_as_uint(xb[3])));
+            }
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) {
+                const bf16x8_t v0 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + lane]);
+                const bf16x8_t v1 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + 64 + lane]);
+                o[2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, ph, o[2 * kk], 0, 0, 0);
+                o[2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, ph, o[2 * kk + 1], 0, 0, 0);
+                o[2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, pl, o[2 * kk], 0, 0, 0);
+                o[2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, pl, o[2 * kk + 1], 0, 0, 0);
+            }
+        }
+        if (F & 4) store(kv_lds + ((step + 1) & 1) * BUF_U4);
+        if (F & 2) __syncthreads();
+    }
+    float acc = l_run;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) acc += o[c][0] + o[c][1] + o[c][2] + o[c][3];
+    out[blockIdx.x * 512 + tid] = acc;
+}
+
+template <int F>
+void run_step(int id, const uint4 *pool, const int *table, float *out, const char *what) {
+    CK(hipFuncSetAttribute(reinterpret_cast<const void *>(&skel<F>), hipFuncAttributeMaxDynamicSharedMemorySize, STEP_LDS_BYTES));
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    float best = 1e9f, sum = 0.f;
+    for (int it = 0; it < 7; ++it) {
+        CK(hipEventRecord(e0));
+        hipLaunchKernelGGL((skel<F>), dim3(256), dim3(512), STEP_LDS_BYTES, 0, pool, table, out, 128);
+        CK(hipEventRecord(e1));
+        CK(hipEventSynchronize(e1));
+        float ms;
+        CK(hipEventElapsedTime(&ms, e0, e1));
+        if (it >= 1) {
+            best = ms < best ? ms : best;
+            sum += ms;
+        }
+    }
+    const double flop = 2.0 * 4 * 256.0 * 128 * 256 * 32 * 256;
+    printf("%d %-66s avg %6.1f us  min %6.1f us  %5.0f TFLOP/s issued (min)\n", id, what, sum / 6 * 1e3, best * 1e3,
+           flop / (best * 1e-3) / 1e12);
+}
+
+template <int T>
+void run(const uint4 *src, float *out, const char *what) {
+    CK(hipFuncSetAttribute(reinterpret_cast<const void *>(&stream<T>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    // 256 workgroups of 128 query slots, 256 page pairs each: 64 products of 32 keys x 32 slots
+    // (or 128 of 16 x 16 ... per tile) per pair and wavefront
+    const int wgs = 256, n_pairs = 256;
+    float best = 1e9f, sum = 0.f;
+    for (int it = 0; it < 7; ++it) {
+        CK(hipEventRecord(e0));
+        hipLaunchKernelGGL((stream<T>), dim3(wgs), dim3(T == 3 ? 512 : 256), LDS_BYTES, 0, src, out, n_pairs);
+        CK(hipEventRecord(e1));
+        CK(hipEventSynchronize(e1));
+        float ms;
+        CK(hipEventElapsedTime(&ms, e0, e1));
+        if (it >= 1) {
+            best = ms < best ? ms : best;
+            sum += ms;
+        }
+    }
+    const double flop = 2.0 * 4 * (double)wgs * 128 * n_pairs * 32 * 256;
+    printf("%d %-66s avg %6.1f us  min %6.1f us  %5.0f TFLOP/s issued (min)\n", T, what, sum / 6 * 1e3, best * 1e3,
+           flop / (best * 1e-3) / 1e12);
+}
+
+int main() {
+    const size_t pool_b = (size_t)2048 * 2048 * 16; // 2048 pages of 32 KiB
+    uint4 *pool;
+    int *table;
+    float *out;
+    CK(hipMalloc(&pool, pool_b));
+    CK(hipMalloc(&table, 2048 * 4));
+    CK(hipMalloc(&out, 256 * 512 * 4));
+    std::vector<int> ht(2048);
+    for (int i = 0; i < 2048; ++i) ht[i] = (i * 977) & 2047;
+    CK(hipMemcpy(table, ht.data(), 2048 * 4, hipMemcpyHostToDevice));
+    std::vector<uint16_t> hp(pool_b / 2);
+    for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 0) {
+            CK(hipMemset(pool, 0x3c, pool_b));
+            printf("== constant operands (every bf16 = 0x3c3c)\n");
+        } else {
+            uint32_t x = 12345;
+            for (auto &h : hp) {
+                x = x * 1664525u + 1013904223u;
+                const float f = ((int)((x >> 8) % 2001u) - 1000) / 4000.0f;
+                uint32_t b;
+                memcpy(&b, &f, 4);
+                h = (uint16_t)(b >> 16);
+            }
+            CK(hipMemcpy(pool, hp.data(), pool_b, hipMemcpyHostToDevice));
+            printf("== random operands in (-0.25, 0.25)\n");
+        }
+        run<0>(pool, out, "32x32x16, operands in registers, 1 wavefront/SIMD");
+        run<1>(pool, out, "32x32x16, A operands from LDS, 1 wavefront/SIMD");
+        run<2>(pool, out, "16x16x32, operands in registers, 1 wavefront/SIMD");
+        run<3>(pool, out, "16x16x32, K and V operands from LDS, 2 wavefronts/SIMD");
+        run_step<1>(4, pool, table, out, "3 + softmax");
+        run_step<3>(5, pool, table, out, "3 + softmax + barrier per four pages");
+        run_step<6>(6, pool, table, out, "3 + barrier + page copies");
+        run_step<7>(7, pool, table, out, "3 + softmax + barrier + page copies (the prefill kernel's step)");
+    }
+    return 0;
+}
