@@ -336,8 +336,9 @@ int32_t skv_attn_gate_device(skv_ctx *ctx, skv_stream stream, const float *ctx_d
  * reference decodes one sequence at a time (encode_resident_full_layer,
  * src/decode_resident/layers.rs:259-288, once per sequence); this is that call applied to
  * a batch, with the same result per sequence. All handles must share the head geometry,
- * the window and the context, and be distinct; nothing is modified when one of them is
- * at capacity. */
+ * the element, the window and the context, and be distinct; nothing is modified when one of
+ * them is at capacity. (One launch pair on either element up to 16 query heads per kv head,
+ * f32 layers up to head_dim 256; other shapes run a launch pair per sequence.) */
 int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_stream stream,
                                      const void *const *k_dev, const void *const *v_dev,
                                      const float *const *q_dev, float *const *out_dev);

@@ -762,7 +762,8 @@ hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t 
     for (int i = 0; i < n_seq; ++i) max_splits = b.seq[i].splits > max_splits ? b.seq[i].splits : max_splits; // == splits_total here
     hipError_t e = hipErrorInvalidValue;
     const bool w8 = a0.waves == 8;
-    switch (a0.g.P) {
+    if (a0.g.f32) e = launch_f32_split_batch(b, n_seq, max_splits, s);
+    else switch (a0.g.P) {
     case 512: e = launch_split_batch<512, 4>(b, n_seq, max_splits, s); break;
     case 32: e = w8 ? launch_split_batch<32, 8>(b, n_seq, max_splits, s) : launch_split_batch<32, 4>(b, n_seq, max_splits, s); break;
     case 64: e = w8 ? launch_split_batch<64, 8>(b, n_seq, max_splits, s) : launch_split_batch<64, 4>(b, n_seq, max_splits, s); break;

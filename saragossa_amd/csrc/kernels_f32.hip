@@ -478,7 +478,7 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
 // page patches its registers from there, so nothing is read back in this launch.
 // ------------------------------------------------------------------------------------
 template <int P, int WAVES, bool PRE>
-__global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
+__device__ __forceinline__ void f32_decode_body(const DecodeArgs &a, const int split, const int kvh) {
     constexpr int NT = P / 16;
     constexpr int THREADS = WAVES * 64;
     extern __shared__ __attribute__((aligned(16))) float4_t lds8[];
@@ -494,12 +494,10 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int j = lane >> 4;
-    const int split = blockIdx.x;
-    const int kvh = blockIdx.y;
     const int G = g.gqa;
     const int n_slots = G; // one query row
     const int q_stride = a.q_head_stride > 0 ? a.q_head_stride : g.head_dim;
-    const int slot0 = blockIdx.z * 16;
+    constexpr int slot0 = 0; // at most 16 heads per group: one tile of query slots
     const int my_limit = min(a.q_pos0, a.limit_cap);
     const int my_ws = a.window > 0 ? max(a.window_start, a.q_pos0 + 1 - a.window) : a.window_start;
 
@@ -843,9 +841,27 @@ __global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
 }
 
 template <int P, int WAVES, bool PRE>
+__global__ __launch_bounds__(WAVES * 64) void f32_decode_kernel(DecodeArgs a) {
+    f32_decode_body<P, WAVES, PRE>(a, blockIdx.x, blockIdx.y);
+}
+
+// Several independent sequences of the same model layer in one launch: grid z is the
+// sequence, grid x covers the largest split count and the others leave early.
+template <int P, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void f32_decode_batch_kernel(DecodeBatchArgs b) {
+    const DecodeArgs &a = b.seq[blockIdx.z];
+    if ((int)blockIdx.x >= a.splits) return;
+    f32_decode_body<P, WAVES, false>(a, blockIdx.x, blockIdx.y);
+}
+
+template <int P, int WAVES>
+constexpr size_t f32_decode_lds() {
+    return (size_t)((P / 16) * 64 + WAVES * (P / 16) * 64) * sizeof(float4_t) + (2 * WAVES * 16 + 2 * P) * sizeof(float);
+}
+
+template <int P, int WAVES, bool PRE>
 static hipError_t launch_f32_decode_pre(const DecodeArgs &a, dim3 grid, hipStream_t s) {
-    constexpr int NT = P / 16;
-    constexpr size_t lds = (size_t)(NT * 64 + WAVES * NT * 64) * sizeof(float4_t) + (2 * WAVES * 16 + 2 * P) * sizeof(float);
+    constexpr size_t lds = f32_decode_lds<P, WAVES>();
     static_assert(lds <= 160 * 1024, "queries and the wavefronts' states share the LDS of a compute unit");
     static std::atomic<uint64_t> lds_ok{0}; // per instantiation
     {
@@ -894,6 +910,36 @@ hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s) {
     case 128: return launch_f32<128>(a, grid, s);
     case 256: return launch_f32<256>(a, grid, s);
     case 512: return launch_f32<512>(a, grid, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <int P, int WAVES>
+static hipError_t launch_f32_batch(const DecodeBatchArgs &b, int n_seq, int max_splits, hipStream_t s) {
+    constexpr size_t lds = f32_decode_lds<P, WAVES>();
+    static std::atomic<uint64_t> lds_ok{0}; // per instantiation
+    {
+        hipError_t e = allow_full_lds(reinterpret_cast<const void *>(&f32_decode_batch_kernel<P, WAVES>), lds_ok);
+        if (e != hipSuccess) return e;
+    }
+    dim3 grid((unsigned)max_splits, (unsigned)b.seq[0].g.kv_heads, (unsigned)n_seq);
+    hipLaunchKernelGGL((f32_decode_batch_kernel<P, WAVES>), grid, dim3(WAVES * 64), lds, s, b);
+    return hipGetLastError();
+}
+
+// The split launch of a batch of f32 sequences (one query row each, every sequence a shape
+// f32_decode_kernel_serves accepts, one geometry; the wavefront count of the first sequence
+// serves all, as in the bf16 batch launch); the caller merges.
+hipError_t launch_f32_split_batch(const DecodeBatchArgs &b, int n_seq, int max_splits, hipStream_t s) {
+    const DecodeArgs &a0 = b.seq[0];
+    for (int i = 0; i < n_seq; ++i)
+        if (!f32_decode_kernel_serves(b.seq[i]) || b.seq[i].pre) return hipErrorInvalidValue;
+    const bool w8 = a0.waves == 8;
+    switch (a0.g.P) {
+    case 32: return w8 ? launch_f32_batch<32, 8>(b, n_seq, max_splits, s) : launch_f32_batch<32, 4>(b, n_seq, max_splits, s);
+    case 64: return w8 ? launch_f32_batch<64, 8>(b, n_seq, max_splits, s) : launch_f32_batch<64, 4>(b, n_seq, max_splits, s);
+    case 128: return w8 ? launch_f32_batch<128, 8>(b, n_seq, max_splits, s) : launch_f32_batch<128, 4>(b, n_seq, max_splits, s);
+    case 256: return w8 ? launch_f32_batch<256, 8>(b, n_seq, max_splits, s) : launch_f32_batch<256, 4>(b, n_seq, max_splits, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -1437,7 +1437,7 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
                                                " atteinte (overflow), séquence " + std::to_string(i));
     }
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(seqs[0]) || seqs[0]->g.gqa > 16 || n_seq == 1 || seqs[0]->g.f32) {
+    if (!fused || !uses_flash(seqs[0]) || seqs[0]->g.gqa > 16 || n_seq == 1 || !fused_append_built(seqs[0])) {
         for (size_t i = 0; i < n_seq; ++i) {
             int32_t rc = skv_decode_step_device(seqs[i], stream, k_dev[i], 0, v_dev[i], 0, q_dev[i], out_dev[i]);
             if (rc) return rc;

@@ -331,6 +331,7 @@ hipError_t launch_f32_split(const DecodeArgs &a, hipStream_t s);
 bool f32_decode_kernel_serves(const DecodeArgs &a); // the launch takes the kernel that can also append the row
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s);
 hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t s);
+hipError_t launch_f32_split_batch(const DecodeBatchArgs &b, int n_seq, int max_splits, hipStream_t s);
 hipError_t launch_merge(const DecodeArgs &a, hipStream_t s);        // split-K partials -> context
 hipError_t launch_prefill_tiles(const DecodeArgs &a, hipStream_t s); // chunked prefill, no merge
 int prefill_tile_slots(int P, bool two_tiles);

@@ -214,12 +214,23 @@ def test_fused_decode_steps_on_f32_layers(state, dims, start, window):
     assert np.array_equal(gk, cache.keys()[n - keep:]) and np.array_equal(gv, cache.values()[n - keep:])
 
 
-def test_decode_step_batch_on_f32_layers(state):
-    dims = (16, 2, 256)
+@pytest.mark.parametrize("dims,lens,window,steps", [
+    ((16, 2, 256), (50, 700, 3000), 0, 3),          # configs[2]'s heads, lengths far apart
+    ((16, 2, 256), (15, 16, 31, 1), 0, 20),         # page boundaries crossed inside the run
+    ((32, 8, 128), (2047, 5, 333, 900, 64), 0, 4),  # configs[1]'s heads
+    ((8, 8, 64), (200, 40), 0, 5),                  # one head per group
+    ((10, 2, 80), (90, 300, 17), 0, 6),             # padded head_dim, five heads per group
+    ((16, 4, 128), (100, 30, 70), 48, 40),          # rings: the window slides and wraps
+    ((4, 1, 320), (40, 200), 0, 3),                 # head_dim above 256: one launch pair per sequence
+])
+def test_decode_step_batch_on_f32_layers(state, dims, lens, window, steps):
+    """skv_decode_step_batch_device on f32 layers: up to head_dim 256 and 16 heads per group one
+    launch pair appends and attends every sequence (f32_decode_batch_kernel); contexts and the
+    rows the launch stored are checked against the oracle's decode_step per sequence."""
     q_dim, kv_dim = dims[0] * dims[2], dims[1] * dims[2]
-    seqs = [_filled(state, dims, n, seed=n) for n in (50, 700, 3000)]
+    seqs = [_filled(state, dims, n, seed=n, window=window, cap=n + steps + 8) for n in lens]
     rng = np.random.default_rng(3)
-    for _ in range(3):
+    for _ in range(steps):
         rows = [(rng.standard_normal(kv_dim, dtype=np.float32), rng.standard_normal(kv_dim, dtype=np.float32),
                  rng.standard_normal(q_dim, dtype=np.float32)) for _ in seqs]
         dev = [[torch.from_numpy(a).cuda() for a in r] for r in rows]
@@ -230,6 +241,12 @@ def test_decode_step_batch_on_f32_layers(state):
         for (kv, cache, lay, _), (k, v, q), o in zip(seqs, rows, outs):
             want = oracle.decode_step(cache, k, v, q, lay)
             assert np.abs(o.cpu().numpy() - want).max() <= TOL
+    for (kv, cache, lay, _), n0 in zip(seqs, lens):
+        n = kv.len()
+        assert n == n0 + steps
+        keep = min(n, window) if window else n
+        gk, gv = kv.read_rows_f32(n - keep, keep)
+        assert np.array_equal(gk, cache.keys()[n - keep:]) and np.array_equal(gv, cache.values()[n - keep:])
 
 
 def test_head_dim_above_512_is_rejected_loudly(state):
