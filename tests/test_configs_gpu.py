@@ -201,6 +201,57 @@ def test_config4_sliding_window_model_batch1_and_batch4(state):
         assert np.array_equal(gk, caches[0].keys()[first:])
 
 
+def test_config4_batch_of_unequal_sequences_on_f32_layers(state):
+    """configs[4]'s group of six layers with the f32 element (what greedy decoding keeps), four
+    sequences of very different lengths per call: every layer's step for the four of them is one
+    launch pair of the f32 batch kernel (global layer at 65536 rows, rings at different fills)."""
+    qh, kvh, hd, window = 16, 8, 256, 1024
+    kv_dim, q_dim = kvh * hd, qh * hd
+    gen = torch.Generator(device="cuda").manual_seed(44)
+    rng = np.random.default_rng(44)
+    lengths, steps = (65536, 9000, 700, 40), 3
+    seqs = []
+    for rows in lengths:
+        layers, caches, lays = [], [], []
+        for li in range(6):
+            w = 0 if (li + 1) % 6 == 0 else window
+            kv = state.full_attention_f32(rows + steps, qh, kvh, hd, window=w)
+            kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+            lay = oracle.layout(qh, kvh, hd, sliding_window=w)
+            c = oracle.LayerKvCache("f32")
+            k, v = _seed_device(kv, rows if w == 0 else min(window, rows), kv_dim, gen)
+            c.append_batch(k, v, lay)
+            layers.append(kv)
+            caches.append(c)
+            lays.append(lay)
+        seqs.append((layers, caches, lays))
+    n = len(seqs)
+    worst = 0.0
+    for _ in range(steps):
+        for li in range(6):
+            q = torch.randn(n, q_dim, device="cuda", generator=gen)
+            k = torch.randn(n, kv_dim, device="cuda", generator=gen)
+            v = torch.randn(n, kv_dim, device="cuda", generator=gen)
+            o = torch.empty(n, q_dim, device="cuda")
+            skv.encode_decode_step_batch([s[0][li] for s in seqs], _stream(),
+                                         [k[i].data_ptr() for i in range(n)], [v[i].data_ptr() for i in range(n)],
+                                         [q[i].data_ptr() for i in range(n)], [o[i].data_ptr() for i in range(n)])
+            got, qh_, kh_, vh_ = o.cpu().numpy(), q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
+            for i, (_, caches, lays) in enumerate(seqs):
+                want = oracle.decode_step(caches[li], kh_[i], vh_[i], qh_[i], lays[li])
+                worst = max(worst, float(np.abs(got[i] - want).max()))
+    assert worst <= 2e-5
+    for (layers, caches, _), r in zip(seqs, lengths):
+        gk, gv = layers[5].read_rows_f32(r - 10, 10 + steps)
+        assert np.array_equal(gk, caches[5].keys()[r - 10:]) and np.array_equal(gv, caches[5].values()[r - 10:])
+        m = layers[0].len()
+        first = max(0, m - window)
+        gk, _ = layers[0].read_rows_f32(first, m - first)
+        assert np.array_equal(gk, caches[0].keys()[first:])
+        for kv in layers:
+            kv.close()
+
+
 def test_config4_local_layer_chunked_prefill_on_the_ring(state):
     """BASELINE configs[4] local layer (q16/kv8/hd256, window 1024 = the ring's rows exactly):
     a prompt prefilled in 512-row chunks equals the oracle's per-row sliding-window attention,
