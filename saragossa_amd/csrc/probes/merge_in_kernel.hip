@@ -56,7 +56,7 @@ __global__ __launch_bounds__(512) void k(Args a) {
     const int wg = kvh * splits + split;
     const int pb0 = (int)(((long)split * a.n_pages) / splits), pb1 = (int)(((long)(split + 1) * a.n_pages) / splits);
     unsigned acc = 0;
-    const size_t page16 = (size_t)2 * 512;
+    const size_t page16 = (size_t)gridDim.y * 512;
     for (int pb = pb0 + wave; pb < pb1; pb += 8) {
         u32x4 kk[8], vv[8];
         int page = __builtin_amdgcn_readfirstlane(a.table[pb]);
@@ -104,9 +104,10 @@ __global__ __launch_bounds__(512) void k(Args a) {
         for (int i0 = 0; i0 < splits; i0 += 16) {
             float4 v[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) v[i] = ld4<AG>(a.part + ((size_t)(kvh * splits + i0 + i) * 512 + tid) * 4);
+            for (int i = 0; i < 16; ++i) v[i] = ld4<AG>(a.part + ((size_t)(kvh * splits + min(i0 + i, splits - 1)) * 512 + tid) * 4);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
+            for (int i = 0; i < 16; ++i)
+                if (i0 + i < splits) { s.x += v[i].x; s.y += v[i].y; s.z += v[i].z; s.w += v[i].w; }
         }
         *(float4 *)(a.out + ((size_t)kvh * 512 + tid) * 4) = s;
         return;
@@ -203,8 +204,18 @@ __global__ __launch_bounds__(256) void merge_like(const float *part, float *out)
     if ((t >> 4) == 0) out[b * 16 + (t & 15)] = s;
 }
 
-int main() {
-    const int rows = 32768, kv_heads = 2, hd = 256, n_pages = rows / 16, NL = 10, splits = 128;
+// Without arguments: the configs[2] shape (32768 rows, 2 kv heads, 128 splits), all modes.
+// With "rows kv_heads splits" (say 2048 8 16, the workgroup count of a short decode launch or
+// of a ring layer): the plain kernel, the hand-off parts, the last workgroup of each kv head
+// merging, and the two-launch pair.
+int main(int argc, char **argv) {
+    const bool full = argc < 4;
+    const int rows = full ? 32768 : atoi(argv[1]), kv_heads = full ? 2 : atoi(argv[2]), hd = 256, n_pages = rows / 16;
+    const int NL = full ? 10 : 36, splits = full ? 128 : atoi(argv[3]);
+    if (n_pages < 1 || kv_heads < 1 || kv_heads > 8 || splits < 1 || splits * kv_heads > 256) {
+        printf("usage: merge_in_kernel [rows kv_heads(<=8) splits(splits*kv_heads<=256)]\n");
+        return 2;
+    }
     const size_t pool_bytes = (size_t)n_pages * kv_heads * hd * 16 * 2;
     std::vector<u32x4 *> kp(NL), vp(NL);
     std::vector<int *> tb(NL);
@@ -219,8 +230,8 @@ int main() {
     }
     Args a{};
     CK(hipMalloc(&a.part, (size_t)256 * 512 * 16)); CK(hipMalloc(&a.part2, (size_t)64 * 512 * 16));
-    CK(hipMalloc(&a.out, 2 * 512 * 16)); CK(hipMalloc(&a.ctr, 64 * 512)); CK(hipMalloc(&a.xcc_seen, 256 * 4));
-    CK(hipMemset(a.ctr, 0, 64 * 512)); CK(hipMemset(a.out, 0, 2 * 512 * 16)); CK(hipMemset(a.xcc_seen, 0xff, 1024));
+    CK(hipMalloc(&a.out, 8 * 512 * 16)); CK(hipMalloc(&a.ctr, 64 * 512)); CK(hipMalloc(&a.xcc_seen, 256 * 4));
+    CK(hipMemset(a.ctr, 0, 64 * 512)); CK(hipMemset(a.out, 0, 8 * 512 * 16)); CK(hipMemset(a.xcc_seen, 0xff, 1024));
     a.n_pages = n_pages;
     hipEvent_t e0, e1;
     CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
@@ -246,24 +257,39 @@ int main() {
         fflush(stdout);
     };
     auto check_out = [&](const char *what) {
-        std::vector<float> h(2 * 512 * 4);
+        std::vector<float> h(8 * 512 * 4);
         CK(hipMemcpy(h.data(), a.out, h.size() * 4, hipMemcpyDeviceToHost));
-        // kv head 0: sum of 1..128 = 8256 ; kv head 1: sum of 129..256 = 24640
+        // kv head h: the sum of its workgroups' values h * splits + 1 .. (h + 1) * splits
         int bad = 0;
-        for (int i = 0; i < 2048; ++i) bad += h[i] != 8256.f;
-        for (int i = 2048; i < 4096; ++i) bad += h[i] != 24640.f;
+        for (int kh = 0; kh < kv_heads; ++kh) {
+            float want = 0.f;
+            for (int i = 0; i < splits; ++i) want += (float)(kh * splits + i + 1);
+            for (int i = 0; i < 2048; ++i) bad += h[kh * 2048 + i] != want;
+        }
         printf("   %s: out[0]=%.0f out[2048]=%.0f mismatches=%d\n", what, h[0], h[2048], bad);
-        CK(hipMemset(a.out, 0, 2 * 512 * 16));
+        CK(hipMemset(a.out, 0, 8 * 512 * 16));
     };
 #define RUN(M, NAME) timeit(NAME, [&](int l) { Args b = a; b.kpool = kp[l]; b.vpool = vp[l]; b.table = tb[l]; \
         hipLaunchKernelGGL(k<M>, dim3(splits, kv_heads), dim3(512), 0, 0, b); });
+    printf("%d rows, %d kv heads x %d splits\n", rows, kv_heads, splits);
     RUN(0, "0 nontemporal partial store, end")
     RUN(1, "1 agent-scope stores + wait + barrier")
-    RUN(2, "2 ... + agent atomic, one counter (256 arrivals)")
-    RUN(3, "3 ... + agent atomic, counter per 16 workgroups")
+    if (full) {
+        RUN(2, "2 ... + agent atomic, one counter (256 arrivals)")
+        RUN(3, "3 ... + agent atomic, counter per 16 workgroups")
+    }
     RUN(4, "4 ... + agent atomic, own counter")
-    RUN(5, "5 one level far: last of 128 merges")
+    RUN(5, "5 one level far: the last workgroup of a kv head merges")
     check_out("mode 5");
+    if (!full) {
+        timeit("pair: mode 0 + merge_like launch", [&](int l) {
+            Args b = a; b.kpool = kp[l]; b.vpool = vp[l]; b.table = tb[l];
+            hipLaunchKernelGGL(k<0>, dim3(splits, kv_heads), dim3(512), 0, 0, b);
+            hipLaunchKernelGGL(merge_like, dim3(256), dim3(256), 0, 0, a.part, a.out);
+        });
+        CK(hipDeviceSynchronize());
+        return 0;
+    }
     RUN(6, "6 two levels far: 16 then 8")
     check_out("mode 6");
     RUN(7, "7 plain stores + L2-scope atomic per (kvh, xcc)")
