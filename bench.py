@@ -703,16 +703,28 @@ def main() -> int:
             for _ in layers:
                 state.encode_probe_empty_launch(stream)
 
+        def read_then_merge_all():
+            # the launch pair of a layer with nothing multiplied: the read-only launch, then the
+            # merge launch of a decode step over the partials the last attention call left
+            for li, kv in enumerate(layers):
+                kv.encode_probe_read_pages(stream)
+                kv.encode_probe_merge(stream, out_arr[li])
+
         read_us = timed_launches(read_all, layers_n)
         empty_us = timed_launches(empty_all, layers_n)
+        pair_us = timed_launches(read_then_merge_all, layers_n)
         kv_bytes = sum(2 * min(kv.len(), kv.window() or kv.len()) * kv_dim * ELEM_BYTES for kv in layers) // layers_n
         ceiling = {"read_only_launch_us": round(read_us, 2),
                    "read_only_gbps": round(kv_bytes / read_us / 1e3, 1),
                    "read_only_frac_of_peak": round(kv_bytes / read_us / 1e3 / HBM_PEAK_GBPS, 4),
                    "empty_launch_us": round(empty_us, 2),
                    "attention_vs_read_only": round(read_us / kern_avg_us, 3),
+                   "read_then_merge_launch_pair_us": round(pair_us, 2),
+                   "attention_vs_read_then_merge": round(pair_us / kern_avg_us, 3),
                    "note": "a launch per layer that only fetches the cached K/V pages with the decode "
-                           "kernel's grid and access pattern (no products, no partials, no merge)"}
+                           "kernel's grid and access pattern (no products, no partials, no merge); "
+                           "read_then_merge: that launch followed by the merge launch of a decode step, "
+                           "the pair of dependent launches an attention call cannot be cheaper than"}
     # the dominant launch is a layer of the first group; with mixed groups the event pairs span
     # all layers, so bytes are summed over the layers and divided by the same time
     late = total_steps + args.steps // 2

@@ -371,6 +371,11 @@ int32_t skv_gather_device(skv_layer *layer, skv_stream stream, size_t first, siz
  * non-temporal loads of whole tiles) and does nothing with them: what a launch that only
  * had to fetch the cache would cost. Async on `stream`. */
 int32_t skv_probe_read_pages_device(skv_layer *layer, skv_stream stream);
+/* The merge launch of a decode step at the layer's current length, over whatever split
+ * partials the layer's buffers hold (those of its last attention call), into out_dev
+ * (q_heads * head_dim f32): behind skv_probe_read_pages_device it is what a decode launch pair
+ * costs when nothing is multiplied. Nothing is launched when the step would take one split. */
+int32_t skv_probe_merge_device(skv_layer *layer, skv_stream stream, float *out_dev);
 /* An empty kernel with the decode launch's shape: the cost of a launch alone. */
 int32_t skv_probe_empty_launch_device(skv_ctx *ctx, skv_stream stream);
 

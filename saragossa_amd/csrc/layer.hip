@@ -1611,6 +1611,19 @@ int32_t skv_probe_read_pages_device(skv_layer *L, skv_stream stream) try {
     return skv::fail_exception();
 }
 
+int32_t skv_probe_merge_device(skv_layer *L, skv_stream stream, float *out_dev) try {
+    if (!L || !out_dev) return fail(SKV_ERR_DEVICE, "probe: pointeur nul");
+    if (L->len == 0) return fail(SKV_ERR_DIMENSION, "probe: cache vide");
+    if (!uses_flash(L)) return fail(SKV_ERR_CONFIG, "probe: noyau matriciel seulement");
+    DecodeArgs a{};
+    fill_decode_args(L, nullptr, out_dev, skv_window_start(L->len - 1, L->window), nullptr, nullptr, 1,
+                     decode_target_wgs(), a);
+    if (a.splits > 1) SKV_HIP(launch_merge(a, as_stream(stream)));
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
 int32_t skv_probe_empty_launch_device(skv_ctx *ctx, skv_stream stream) try {
     if (!ctx) return fail(SKV_ERR_DEVICE, "probe: ctx nul");
     SKV_HIP(launch_probe_empty(as_stream(stream)));

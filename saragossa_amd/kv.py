@@ -258,6 +258,11 @@ class FullAttentionState:
         decode kernel's grid and access pattern."""
         check(self._l.skv_probe_read_pages_device(self._h, stream))
 
+    def encode_probe_merge(self, stream, out_ptr) -> None:
+        """Measurement aid: the merge launch of a decode step at the current length, over the
+        partials the layer's last attention call left."""
+        check(self._l.skv_probe_merge_device(self._h, stream, out_ptr))
+
     def encode_decode_step(self, stream, k_ptr, k_off, v_ptr, v_off, q_ptr, out_ptr) -> None:
         check(self._l.skv_decode_step_device(self._h, stream, k_ptr, k_off, v_ptr, v_off, q_ptr,
                                              out_ptr))

@@ -51,6 +51,7 @@ def test_default_run_prints_one_json_line_with_the_agreed_keys():
     cb = d["cpu_baseline"]
     assert cb["kind"] == "port" and cb["unit"] == "us/token" and cb["cores"] >= 1 and cb["value"] > 0
     assert d["ceiling"]["read_only_launch_us"] > 0
+    assert d["ceiling"]["read_then_merge_launch_pair_us"] >= d["ceiling"]["read_only_launch_us"]
 
 
 @pytest.mark.gpu

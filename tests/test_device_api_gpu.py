@@ -317,8 +317,8 @@ def test_attention_launches_replay_correctly_from_a_hip_graph(state):
 
 
 def test_measurement_probes_leave_the_cache_untouched(state):
-    # the read-only and empty launches that the benchmark times beside the attention launch:
-    # they run on full and ring layers at ragged lengths and change nothing
+    # the read-only, merge-only and empty launches that the benchmark times beside the attention
+    # launch: they run on full and ring layers at ragged lengths and change nothing
     rng = np.random.default_rng(31)
     for (q_heads, kv_heads, head_dim), window, n in (((16, 2, 256), None, 1000), ((8, 2, 128), 64, 333),
                                                      ((8, 8, 64), None, 1), ((4, 1, 512), None, 47)):
@@ -333,8 +333,10 @@ def test_measurement_probes_leave_the_cache_untouched(state):
         q = rng.standard_normal(q_heads * head_dim, dtype=np.float32)
         attend = (lambda: kv.attention_decode_windowed(q, first)) if window else (lambda: kv.attention_decode(q))
         want = attend()
+        scratch_out = torch.empty(q_heads * head_dim, device="cuda")
         for _ in range(3):
             kv.encode_probe_read_pages(_stream())
+            kv.encode_probe_merge(_stream(), scratch_out.data_ptr())
             state.encode_probe_empty_launch(_stream())
         torch.cuda.synchronize()
         after = kv.read_rows(first)
