@@ -916,6 +916,7 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
         return fail(SKV_ERR_DIMENSION, "append KV résident: capacité " +
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     // the attention kernel writes the row itself: advance the bookkeeping first
+    const size_t floor_before = L->floor_pos;
     L->len += 1;
     if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
         L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
@@ -923,7 +924,10 @@ int32_t skv_decode_step_device(skv_layer *L, skv_stream stream, const void *k_de
     int32_t rc = encode_attention(L, as_stream(stream), q_dev, out_dev, ws,
                                   reinterpret_cast<const float *>((const char *)k_dev + k_off),
                                   reinterpret_cast<const float *>((const char *)v_dev + v_off));
-    if (rc) L->len -= 1;
+    if (rc) {
+        L->len -= 1;
+        L->floor_pos = floor_before;
+    }
     return rc;
 } catch (...) {
     return skv::fail_exception();
@@ -1455,9 +1459,11 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
             pages_total += (rows + 15) / 16;
         }
         DecodeBatchArgs b{};
+        size_t floor_before[SKV_MAX_BATCH];
         for (size_t i = 0; i < n; ++i) {
             skv_layer *L = seqs[first + i];
             // the attention kernel writes the row itself: advance the bookkeeping first
+            floor_before[i] = L->floor_pos;
             L->len += 1;
             if (L->g.ring_rows > 0 && L->len > (size_t)L->g.ring_rows)
                 L->floor_pos = std::max(L->floor_pos, L->len - (size_t)L->g.ring_rows);
@@ -1471,7 +1477,10 @@ int32_t skv_decode_step_batch_device(skv_layer *const *seqs, size_t n_seq, skv_s
         }
         hipError_t e = launch_decode_batch(b, (int)n, as_stream(stream));
         if (e != hipSuccess) {
-            for (size_t i = 0; i < n; ++i) seqs[first + i]->len -= 1;
+            for (size_t i = 0; i < n; ++i) {
+                seqs[first + i]->len -= 1;
+                seqs[first + i]->floor_pos = floor_before[i];
+            }
             return fail_hip(e, "decode_step_batch: lancement");
         }
     }
