@@ -195,7 +195,10 @@ int choose_splits(const skv_layer *L, int n_pages_scan, size_t rows, int waves, 
     if (!skv_flag_sdpa_2pass_enabled() || rows < t.split_min_len) return 1;
     const size_t min_pages = std::max<size_t>(t.min_pages ? t.min_pages : (size_t)waves, 1);
     size_t s = std::max<size_t>(target_wgs / (size_t)L->g.kv_heads, 1);
-    s = std::min<size_t>(s, (size_t)n_pages_scan / min_pages);
+    // Short contexts: as many splits as leave no split more than min_pages pages (rounded up,
+    // not down: with one page per wavefront no wavefront then walks a second page, which
+    // would be a whole memory latency more for the launch).
+    s = std::min<size_t>(s, ((size_t)n_pages_scan + min_pages - 1) / min_pages);
     s = std::min<size_t>(s, (size_t)L->max_splits);
     return (int)std::max<size_t>(s, 1);
 }
