@@ -51,6 +51,13 @@ WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {2: 70175 * 1024}
 
 
+# What the matrix pipes sustain for the prefill kernel's product stream when nothing else is in
+# the kernel: 16x16x32 bf16 products with every operand in registers, on random operand values
+# (the clock under the matrix pipes drops when operand bits toggle), measured with the
+# stand-alone program saragossa_amd/csrc/probes/mfma_stream.hip (variant 2) on one MI355X. A
+# recorded figure, like the traffic above; the published peak stays the roofline's `peak`.
+MFMA_STREAM_RANDOM_TFLOPS = 1580.0
+
 ELEM_BYTES = 2  # bytes of a cached K or V element in the decode leg: 2 (bf16) or 4 (--element f32)
 
 
@@ -244,6 +251,7 @@ def bench_prefill(skv, torch, np, state, stream, element="bf16"):
         else:
             row["mfma_tflops_issued"] = round(2 * flops / us / 1e6, 1)
             row["frac_of_bf16_mfma_peak"] = round(2 * flops / us / 1e6 / 2500.0, 4)
+            row["issued_vs_recorded_product_stream"] = round(2 * flops / us / 1e6 / MFMA_STREAM_RANDOM_TFLOPS, 4)
         out.append(row)
         kv.close()
     return out
