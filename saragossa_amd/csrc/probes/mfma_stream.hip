@@ -11,6 +11,8 @@
 //   4-7  variant 3 plus the other parts of the prefill kernel's step: online softmax (4), and the
 //      barrier of every step (5); barrier and page copies through registers into LDS without
 //      the softmax (6); all of them (7)
+//   8  the f32 element's products (16x16x4 f32, operands in registers, two wavefronts per SIMD),
+//      as many flops as the f32 chunk kernel issues for the same chunk (277 GFLOP)
 // Each variant runs twice: on a constant bit pattern and on random values in (-0.25, 0.25). The
 // clock the device sustains under the matrix pipes depends on how many operand bits toggle, so
 // the second figure is the one a kernel on real data can be held against.
@@ -297,6 +299,51 @@ void run_step(int id, const uint4 *pool, const int *table, float *out, const cha
            flop / (best * 1e-3) / 1e12);
 }
 
+// The f32 element's products: v_mfma_f32_16x16x4_f32 with every operand in registers, two
+// wavefronts per SIMD, as many flops as the f32 chunk issues (no second term: 277 GFLOP).
+__global__ __launch_bounds__(512) void stream_f32(const uint4 *src, float *out, int n_iter) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    float q[32];
+#pragma unroll
+    for (int s = 0; s < 32; ++s) q[s] = __uint_as_float(src[(s * 64 + lane) & 4095].x) * 1e-3f;
+    float4_t acc[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < n_iter; ++it) {
+#pragma unroll
+        for (int s = 0; s < 128; ++s)
+            acc[s & 7] = __builtin_amdgcn_mfma_f32_16x16x4f32(q[s & 31], q[(s + 5) & 31], acc[s & 7], 0, 0, 0);
+    }
+    float r = 0.f;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) r += acc[b][0] + acc[b][1] + acc[b][2] + acc[b][3];
+    out[blockIdx.x * blockDim.x + tid] = r;
+}
+
+void run_f32(const uint4 *src, float *out) {
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    // 256 workgroups x 8 wavefronts x n_iter x 128 products of 2048 flops
+    const int n_iter = 516;
+    float best = 1e9f, sum = 0.f;
+    for (int it = 0; it < 7; ++it) {
+        CK(hipEventRecord(e0));
+        hipLaunchKernelGGL(stream_f32, dim3(256), dim3(512), 0, 0, src, out, n_iter);
+        CK(hipEventRecord(e1));
+        CK(hipEventSynchronize(e1));
+        float ms;
+        CK(hipEventElapsedTime(&ms, e0, e1));
+        if (it >= 1) {
+            best = ms < best ? ms : best;
+            sum += ms;
+        }
+    }
+    const double flop = 256.0 * 8 * n_iter * 128 * 2048;
+    printf("8 %-66s avg %6.1f us  min %6.1f us  %5.1f TFLOP/s (min)\n", "f32 16x16x4, operands in registers, 2 wavefronts/SIMD", sum / 6 * 1e3,
+           best * 1e3, flop / (best * 1e-3) / 1e12);
+}
+
 template <int T>
 void run(const uint4 *src, float *out, const char *what) {
     CK(hipFuncSetAttribute(reinterpret_cast<const void *>(&stream<T>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES));
@@ -360,6 +407,7 @@ int main() {
         run_step<3>(5, pool, table, out, "3 + softmax + barrier per four pages");
         run_step<6>(6, pool, table, out, "3 + barrier + page copies");
         run_step<7>(7, pool, table, out, "3 + softmax + barrier + page copies (the prefill kernel's step)");
+        run_f32(pool, out);
     }
     return 0;
 }
