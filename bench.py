@@ -593,7 +593,7 @@ def main() -> int:
     for n, _, _, _, rows, window in groups:
         for _ in range(n):
             for _ in range(B):   # every sequence owns its pages and its block table
-                kv = state.full_attention_with_element(rows + 2 * total_steps + 8, qh, kvh, hd,
+                kv = state.full_attention_with_element(rows + 3 * total_steps + 8, qh, kvh, hd,
                                                        skv.DTYPE_F32 if args.element == "f32" else skv.DTYPE_BF16,
                                                        window)
                 kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
@@ -608,7 +608,10 @@ def main() -> int:
                 layers.append(kv)
             layer_rows.append(fill)
 
-    n_pass = 2 * total_steps  # timed pass + per-kernel pass
+    # the ring layers between two global layers share a geometry: a caller that holds the q/k/v of
+    # several of them at once can step them in one launch pair (informational leg, see below)
+    grouped_leg = B == 1 and any(g[5] for g in groups) and any(not g[5] for g in groups)
+    n_pass = (3 if grouped_leg else 2) * total_steps  # timed pass + per-kernel pass (+ grouped pass)
     n_units = layers_n * B   # (layer, sequence) pairs, layer-major
     q_all = torch.randn(n_pass, n_units, q_dim, device=dev, dtype=torch.float32, generator=gen)
     k_all = torch.randn(n_pass, n_units, kv_dim, device=dev, dtype=torch.float32, generator=gen)
@@ -733,6 +736,58 @@ def main() -> int:
                            "kernel's grid and access pattern (no products, no partials, no merge); "
                            "read_then_merge: that launch followed by the merge launch of a decode step, "
                            "the pair of dependent launches an attention call cannot be cheaper than"}
+    grouped = None
+    if grouped_leg:
+        # Informational, never `value`: the same token with the ring layers stepped five at a time
+        # through skv_decode_step_batch_device (handles of one geometry and window, here layers
+        # instead of sequences), the global layers one by one as before. Only a caller that holds
+        # the q/k/v of those five layers at once can do this; a decoder whose layer l+1 consumes
+        # layer l's output cannot, which is why the headline figure does not.
+        windows = [g[5] for g in groups for _ in range(g[0])]
+        ring_ix = [i for i, w in enumerate(windows) if w]
+        glob_ix = [i for i, w in enumerate(windows) if not w]
+        per_call = 5
+        n_glob = len(glob_ix)
+        GArr = C.c_void_p * n_glob
+
+        def pick(arr, ix):
+            return (C.c_void_p * len(ix))(*[arr[i] for i in ix])
+
+        glob_layers = pick(layer_arr, glob_ix)
+        glob_out = pick(out_arr, glob_ix)
+        ring_calls = [ring_ix[i:i + per_call] for i in range(0, len(ring_ix), per_call)]
+        ring_layers = [pick(layer_arr, ix) for ix in ring_calls]
+        ring_out = [pick(out_arr, ix) for ix in ring_calls]
+
+        def run_grouped(st):
+            kp, vp, qp = step_ptrs[st]
+            rc = lib.skv_decode_step_layers_device(glob_layers, n_glob, stream, pick(kp, glob_ix), pick(vp, glob_ix),
+                                                   pick(qp, glob_ix), glob_out)
+            if rc:
+                raise RuntimeError(lib.skv_last_error().decode())
+            for ix, la, oa in zip(ring_calls, ring_layers, ring_out):
+                rc = lib.skv_decode_step_batch_device(la, len(ix), stream, pick(kp, ix), pick(vp, ix), pick(qp, ix), oa)
+                if rc:
+                    raise RuntimeError(lib.skv_last_error().decode())
+
+        base_step = 2 * total_steps
+        for st in range(base_step, base_step + args.warmup):
+            run_grouped(st)
+        torch.cuda.synchronize()
+        g0 = time.perf_counter()
+        for st in range(base_step + args.warmup, base_step + total_steps):
+            run_grouped(st)
+        torch.cuda.synchronize()
+        g_us = (time.perf_counter() - g0) * 1e6 / args.steps
+        g_mid = base_step + args.warmup + args.steps // 2
+        g_bytes = sum(algorithmic_bytes(min(r + g_mid, w) if w else r + g_mid, kv_dim, q_dim, True)
+                      for r, w in zip(layer_rows, windows))
+        grouped = {"us_per_token": round(g_us, 2), "hbm_frac": round(g_bytes / g_us / 1e3 / HBM_PEAK_GBPS, 4),
+                   "ring_layers_per_launch_pair": per_call,
+                   "note": "informational, not `value`: the ring layers stepped five per launch pair through "
+                           "skv_decode_step_batch_device, which needs the q/k/v of those layers at once; a "
+                           "decoder whose next layer consumes this layer's output cannot call it that way"}
+
     # the dominant launch is a layer of the first group; with mixed groups the event pairs span
     # all layers, so bytes are summed over the layers and divided by the same time
     late = total_steps + args.steps // 2
@@ -827,6 +882,8 @@ def main() -> int:
     }
     if ceiling is not None:
         result["ceiling"] = ceiling
+    if grouped is not None:
+        result["ring_layers_batched"] = grouped
     if restore is not None:
         result["restore"] = restore
     if recurrent is not None:
