@@ -53,9 +53,9 @@ MEASURED_TRAFFIC_BYTES = {2: 70175 * 1024}
 
 # What the matrix pipes sustain for the prefill kernel's product stream when nothing else is in
 # the kernel: 16x16x32 bf16 products with every operand in registers, on random operand values
-# (the clock under the matrix pipes drops when operand bits toggle), measured with the
-# stand-alone program saragossa_amd/csrc/probes/mfma_stream.hip (variant 2) on one MI355X. A
-# recorded figure, like the traffic above; the published peak stays the roofline's `peak`.
+# (the clock under the matrix pipes drops when operand bits toggle), measured once with a
+# stand-alone product-stream program on one MI355X. A recorded figure, like the traffic above;
+# the published peak stays the roofline's `peak`.
 MFMA_STREAM_RANDOM_TFLOPS = 1580.0
 
 ELEM_BYTES = 2  # bytes of a cached K or V element in the decode leg: 2 (bf16) or 4 (--element f32)
