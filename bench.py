@@ -58,15 +58,13 @@ MEASURED_TRAFFIC_BYTES = {2: 70175 * 1024}
 # the published peak stays the roofline's `peak`.
 MFMA_STREAM_RANDOM_TFLOPS = 1580.0
 
-ELEM_BYTES = 2  # bytes of a cached K or V element in the decode leg: 2 (bf16) or 4 (--element f32)
-
-
-def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool) -> int:
-    """Bytes one layer's decode step has to move: K and V once (in the cache's element), q in
-    and ctx out (f32), the block table, and the appended row when the append is counted."""
-    b = 2 * rows * kv_dim * ELEM_BYTES + 2 * q_dim * 4 + (rows + 15) // 16 * 4
+def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool, elem_bytes: int = 2) -> int:
+    """Bytes one layer's decode step has to move: K and V once (in the cache's element: 2 bytes
+    for bf16, 4 for f32), q in and ctx out (f32), the block table, and the appended row when the
+    append is counted."""
+    b = 2 * rows * kv_dim * elem_bytes + 2 * q_dim * 4 + (rows + 15) // 16 * 4
     if with_append:
-        b += 2 * kv_dim * ELEM_BYTES
+        b += 2 * kv_dim * elem_bytes
     return b
 
 
@@ -345,6 +343,35 @@ def config3_traffic(np):
     return shared, hist, turn
 
 
+def restore_cpu_baseline(np, seconds):
+    """The reference's CPU path at the prefix-cache boundary: remember_prefix_block clones the whole
+    f32 prompt state (src/serve/state.rs:613-639) and match_prefix clones the hit's state
+    (src/serve/cache.rs:121-151). The oracle's state clone is a deep copy of [n, kv_dim] f32 K and
+    V per layer; timed here for the 4096-token boundary of configs[3] (36 layers, kv8/hd128), a
+    bounded sample scaled to the 36 layers."""
+    import oracle
+    qh, kvh, hd, nl, n = 32, 8, 128, 36, 4096
+    kv_dim = kvh * hd
+    k = np.ones((n, kv_dim), np.float32)
+    caches = []
+    for _ in range(4):
+        c = oracle.LayerKvCache("f32")
+        c.append_batch(k, k, oracle.layout(qh, kvh, hd))
+        caches.append(c)
+    c0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - c0 < seconds:
+        for c in caches:
+            c.clone()
+        reps += 1
+    dt = (time.perf_counter() - c0) / reps / len(caches) * nl
+    payload_f32 = n * kv_dim * 4 * 2 * nl
+    return {"value": round(payload_f32 / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "deep copy of one layer's f32 K/V at 4096 rows, %d x 4 copies timed, scaled to %d "
+                      "layers: %.1f ms per cloned 4096-token state (the reference clones one per block "
+                      "boundary and one per hit)" % (reps, nl, dt * 1e3)}
+
+
 def bench_config3(args, skv, torch, np, state, stream):
     """BASELINE.json configs[3]: 8 sessions share a 4096-token prefix, each adds a 256..1024
     token history and then a 512-token turn; 16-token hash blocks over 36 layers of Qwen3-4B
@@ -500,31 +527,7 @@ def bench_config3(args, skv, torch, np, state, stream):
     for kv in proto + layers:
         kv.close()
     if not args.no_cpu_baseline:
-        # The reference's CPU path at the same boundary: remember_prefix_block clones the whole
-        # f32 prompt state (src/serve/state.rs:613-639) and match_prefix clones the hit's state
-        # (src/serve/cache.rs:121-151). The oracle's state clone is a deep copy of [n, kv_dim]
-        # f32 K and V per layer; timed here for the 4096-token boundary, a bounded sample.
-        import oracle
-        n = 4096
-        k = np.ones((n, kv_dim), np.float32)
-        caches = []
-        for _ in range(4):
-            c = oracle.LayerKvCache("f32")
-            c.append_batch(k, k, oracle.layout(qh, kvh, hd))
-            caches.append(c)
-        c0 = time.perf_counter()
-        reps = 0
-        while time.perf_counter() - c0 < min(args.cpu_seconds, 10.0):
-            for c in caches:
-                c.clone()
-            reps += 1
-        dt = (time.perf_counter() - c0) / reps / len(caches) * nl
-        payload_f32 = n * kv_dim * 4 * 2 * nl
-        result["cpu_baseline"] = {
-            "value": round(payload_f32 / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "deep copy of one layer's f32 K/V at 4096 rows, %d x 4 copies timed, scaled to %d "
-                      "layers: %.1f ms per cloned 4096-token state (the reference clones one per block "
-                      "boundary and one per hit)" % (reps, nl, dt * 1e3)}
+        result["cpu_baseline"] = restore_cpu_baseline(np, min(args.cpu_seconds, 10.0))
     print(json.dumps(result))
     return 0
 
@@ -542,7 +545,9 @@ def main() -> int:
                     help="element of the decode leg's caches (f32 is the reference's choice for greedy decoding)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-restore", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=3.0)
+    ap.add_argument("--no-legs", action="store_true",
+                    help="default run only: skip the configs[4] batch-4 and f32-element legs")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--end-to-end", action="store_true",
                     help="with --config 1: also run the whole random-init decoder and report tok/s")
     args = ap.parse_args()
@@ -559,16 +564,57 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the KV path has no CPU fallback", file=sys.stderr)
         return 2
-    global ELEM_BYTES
-    ELEM_BYTES = 4 if args.element == "f32" else 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.config == 3:
         return bench_config3(args, skv, torch, np, skv.DecodeResidentState(0),
                              torch.cuda.current_stream().cuda_stream)
+    if args.batch < 1:
+        print("bench.py: --batch must be at least 1", file=sys.stderr)
+        return 2
+    state = skv.DecodeResidentState(0)
+    result = decode_bench(args, skv, torch, np, state, main_leg=True)
+    if args.config == 2 and args.batch == 1 and args.element == "bf16" and not args.context and not args.no_legs:
+        # Further legs of the default run, each timed like the headline and reported with its own
+        # roofline object: BASELINE configs[4] at batch 4 (one launch pair per layer covers the
+        # four sequences) and configs[2] on the cache's f32 element (the reference's choice for
+        # greedy decoding). Fewer steps than the headline: they only have to be steady.
+        import argparse as _ap
+        legs = {}
+        for key, over in (("configs4_batch4", dict(config=4, batch=4, element="bf16", steps=min(args.steps, 32), warmup=4)),
+                          ("configs2_f32_element", dict(config=2, batch=1, element="f32", steps=min(args.steps, 64), warmup=4))):
+            ns = _ap.Namespace(**vars(args))
+            for k, v in over.items():
+                setattr(ns, k, v)
+            ns.no_cpu_baseline = True
+            leg = decode_bench(ns, skv, torch, np, state, main_leg=False)
+            legs[key] = {k: leg[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "dtype", "config",
+                                             "tok_per_s", "hbm_gbps", "hbm_frac", "roofline", "checked_max_abs")
+                         if k in leg}
+            if "ceiling" in leg:
+                legs[key]["ceiling"] = leg["ceiling"]
+        result["legs"] = legs
+    print(json.dumps(result))
+    return 0
+
+
+def decode_bench(args, skv, torch, np, state, main_leg):
+    """One decode workload (args.config, args.batch, args.element): builds the caches, times
+    args.steps steps after args.warmup, checks the last context against float64 softmax
+    attention, times the attention launches with HIP events, and returns the result object.
+    The restore, recurrent-state, prefill and CPU legs only run for the main leg."""
+    import ctypes as C
+    dev = torch.device("cuda:0")
+    ELEM_BYTES = 4 if args.element == "f32" else 2
+
+    def algorithmic(rows, kv_dim_, q_dim_, with_append):
+        return algorithmic_bytes(rows, kv_dim_, q_dim_, with_append, ELEM_BYTES)
+
     wl = WORKLOADS[args.config]
+    no_cpu = args.no_cpu_baseline or not main_leg
+    no_restore = args.no_restore or not main_leg
     if len(wl["groups"]) > 1:
-        args.no_cpu_baseline = True   # the CPU sample is scaled by identical layers only
+        no_cpu = True   # the CPU sample is scaled by identical layers only
     groups = [(n, qh_, kvh_, hd_, args.context or ctx_, w_) for n, qh_, kvh_, hd_, ctx_, w_ in wl["groups"]]
     qh, kvh, hd = groups[0][1:4]     # all groups of a workload share the head shape
     kv_dim, q_dim = kvh * hd, qh * hd
@@ -579,14 +625,10 @@ def main() -> int:
     gen = torch.Generator(device=dev)
     gen.manual_seed(args.config)
     rng = np.random.default_rng(args.config)
-    state = skv.DecodeResidentState(0)
     stream = torch.cuda.current_stream().cuda_stream
     B = args.batch
-    if B < 1:
-        print("bench.py: --batch must be at least 1", file=sys.stderr)
-        return 2
     if B > 1:
-        args.no_cpu_baseline = True   # the CPU sample is one sequence
+        no_cpu = True   # the CPU sample is one sequence
     layers = []       # one handle per (layer, sequence), layer-major
     layer_rows = []   # rows each layer attends per step (for the byte count)
     host_kv = []      # first layer's f32 rows, kept for the CPU baseline
@@ -602,7 +644,7 @@ def main() -> int:
                 v = torch.randn(fill, kv_dim, device=dev, dtype=torch.float32, generator=gen)
                 kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), fill)
                 torch.cuda.synchronize()
-                if not layers and not args.no_cpu_baseline:
+                if not layers and not no_cpu:
                     host_kv = [k.cpu().numpy(), v.cpu().numpy()]
                 del k, v
                 layers.append(kv)
@@ -657,9 +699,26 @@ def main() -> int:
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     step_us = ms_per_step * 1e3
+    # Proof that the timed kernels did the work: the context the last timed step left for layer 0
+    # (sequence 0), against textbook softmax attention in float64 (torch, on the device) over the
+    # rows read back from that layer's cache; shares nothing with the library's kernels or the
+    # CPU oracle.
+    kv0 = layers[0]
+    gk, gv = kv0.read_rows_f32()
+    n0 = gk.shape[0]
+    Kd = torch.from_numpy(gk).to(dev).double().view(n0, kvh, hd)
+    Vd = torch.from_numpy(gv).to(dev).double().view(n0, kvh, hd)
+    qd = q_all[total_steps - 1, 0].double().view(kvh, qh // kvh, hd)
+    prob = torch.softmax(torch.einsum("kgd,nkd->kgn", qd, Kd) / hd ** 0.5, dim=-1)
+    ref = torch.einsum("kgn,nkd->kgd", prob, Vd).reshape(-1)
+    checked_max_abs = float((out[0].double() - ref).abs().max())
+    del Kd, Vd, prob, ref, gk, gv
+    if not checked_max_abs <= 1e-4:
+        raise RuntimeError("bench: the last timed step's context of layer 0 differs from float64 softmax "
+                           "attention over the cached rows by %.3e (> 1e-4)" % checked_max_abs)
     us_per_token = step_us / B   # a step yields one token per sequence
     mid = args.warmup + args.steps // 2
-    step_bytes = B * sum(algorithmic_bytes(min(r + mid, w) if w else r + mid, kv_dim, q_dim, True)
+    step_bytes = B * sum(algorithmic(min(r + mid, w) if w else r + mid, kv_dim, q_dim, True)
                          for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
 
     # ---- per-kernel pass on the launch stream: the ten appends of a token first, then HIP
@@ -721,9 +780,17 @@ def main() -> int:
                 kv.encode_probe_read_pages(stream)
                 kv.encode_probe_merge(stream, out_arr[li])
 
+        def read_store_then_merge_all():
+            # the same pair when the first launch also leaves a split partial per workgroup, as
+            # any split-K launch must before a merge can run
+            for li, kv in enumerate(layers):
+                kv.encode_probe_read_store_pages(stream)
+                kv.encode_probe_merge(stream, out_arr[li])
+
         read_us = timed_launches(read_all, layers_n)
         empty_us = timed_launches(empty_all, layers_n)
         pair_us = timed_launches(read_then_merge_all, layers_n)
+        pair_store_us = timed_launches(read_store_then_merge_all, layers_n)
         kv_bytes = sum(2 * min(kv.len(), kv.window() or kv.len()) * kv_dim * ELEM_BYTES for kv in layers) // layers_n
         ceiling = {"read_only_launch_us": round(read_us, 2),
                    "read_only_gbps": round(kv_bytes / read_us / 1e3, 1),
@@ -732,10 +799,14 @@ def main() -> int:
                    "attention_vs_read_only": round(read_us / kern_avg_us, 3),
                    "read_then_merge_launch_pair_us": round(pair_us, 2),
                    "attention_vs_read_then_merge": round(pair_us / kern_avg_us, 3),
+                   "read_store_then_merge_launch_pair_us": round(pair_store_us, 2),
+                   "attention_vs_read_store_then_merge": round(pair_store_us / kern_avg_us, 3),
                    "note": "a launch per layer that only fetches the cached K/V pages with the decode "
                            "kernel's grid and access pattern (no products, no partials, no merge); "
                            "read_then_merge: that launch followed by the merge launch of a decode step, "
-                           "the pair of dependent launches an attention call cannot be cheaper than"}
+                           "the pair of dependent launches an attention call cannot be cheaper than; "
+                           "read_store_then_merge: the same with a split partial of the decode kernel's size "
+                           "written by every workgroup of the first launch"}
     grouped = None
     if grouped_leg:
         # Informational, never `value`: the same token with the ring layers stepped five at a time
@@ -780,7 +851,7 @@ def main() -> int:
         torch.cuda.synchronize()
         g_us = (time.perf_counter() - g0) * 1e6 / args.steps
         g_mid = base_step + args.warmup + args.steps // 2
-        g_bytes = sum(algorithmic_bytes(min(r + g_mid, w) if w else r + g_mid, kv_dim, q_dim, True)
+        g_bytes = sum(algorithmic(min(r + g_mid, w) if w else r + g_mid, kv_dim, q_dim, True)
                       for r, w in zip(layer_rows, windows))
         grouped = {"us_per_token": round(g_us, 2), "hbm_frac": round(g_bytes / g_us / 1e3 / HBM_PEAK_GBPS, 4),
                    "ring_layers_per_launch_pair": per_call,
@@ -791,21 +862,23 @@ def main() -> int:
     # the dominant launch is a layer of the first group; with mixed groups the event pairs span
     # all layers, so bytes are summed over the layers and divided by the same time
     late = total_steps + args.steps // 2
-    all_bytes = B * sum(algorithmic_bytes(min(r + late, w) if w else r + late, kv_dim, q_dim, B > 1)
+    all_bytes = B * sum(algorithmic(min(r + late, w) if w else r + late, kv_dim, q_dim, B > 1)
                         for r, w in zip(layer_rows, [g[5] for g in groups for _ in range(g[0])]))
     launch_bytes = all_bytes // layers_n
     achieved = launch_bytes / (kern_avg_us * 1e-6) / 1e9
     cpu_inputs = None
-    if not args.no_cpu_baseline:
+    if not no_cpu:
         cpu_inputs = (k_all[:, 0].cpu().numpy(), v_all[:, 0].cpu().numpy(), q_all[:, 0].cpu().numpy())
     for kv in layers:
         kv.close()
     del layers, q_all, k_all, v_all
     torch.cuda.empty_cache()
 
-    restore = None if (args.no_restore or args.config != 2) else bench_restore(skv, torch, np, state, stream, args.element)
+    restore = None if (no_restore or args.config != 2) else bench_restore(skv, torch, np, state, stream, args.element)
+    if restore is not None and not no_cpu:
+        restore["cpu_baseline"] = restore_cpu_baseline(np, min(args.cpu_seconds, 10.0))
     recurrent = None
-    if args.config == 2 and not args.no_restore:
+    if args.config == 2 and not no_restore:
         # configs[2]'s 30 linear-attention layers: their recurrent state (conv 96 KiB + ssm 2 MiB
         # each, f32) is snapshotted and restored as flat device-to-device copies
         sizes = [96 * 1024, 2 * 1024 * 1024] * 30
@@ -863,6 +936,9 @@ def main() -> int:
         "tok_per_s": round(1e6 / us_per_token, 1),
         "hbm_gbps": round(step_bytes / (step_us * 1e-6) / 1e9, 1),
         "hbm_frac": round(step_bytes / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "checked_max_abs": checked_max_abs,
+        "checked": "context of layer 0 after the last timed step vs float64 softmax attention (torch) over "
+                   "the rows read back from its cache; the run fails above 1e-4",
         "roofline": {"bound": "hbm", "kernel": ("f32_split_kernel<%d> + decode_merge_kernel (one attention launch per "
                                                 "sequence, average over the layers)" if args.element == "f32" else
                                                 "decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
@@ -888,12 +964,12 @@ def main() -> int:
         result["restore"] = restore
     if recurrent is not None:
         result["recurrent_state"] = recurrent
-    if args.config == 1 and args.end_to_end:
+    if args.config == 1 and args.end_to_end and main_leg:
         result["end_to_end"] = bench_end_to_end(skv, torch, np, state)
-    if args.config == 2 and not args.no_restore:
+    if args.config == 2 and not no_restore:
         result["prefill"] = bench_prefill(skv, torch, np, state, stream, args.element)
 
-    if not args.no_cpu_baseline:
+    if not no_cpu:
         import oracle
         threads = oracle.default_threads(qh)
         lay = oracle.layout(qh, kvh, hd)
@@ -915,9 +991,7 @@ def main() -> int:
             "sample": "%d layer-steps of append + cached_attention_one on layer 0 (f32 cache, "
                       "%d rows) timed and scaled by %d layers; host has %d cores"
                       % (n_calls, ctx_rows, layers_n, os.cpu_count() or 0)}
-
-    print(json.dumps(result))
-    return 0
+    return result
 
 
 if __name__ == "__main__":

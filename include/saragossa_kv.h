@@ -371,6 +371,11 @@ int32_t skv_gather_device(skv_layer *layer, skv_stream stream, size_t first, siz
  * non-temporal loads of whole tiles) and does nothing with them: what a launch that only
  * had to fetch the cache would cost. Async on `stream`. */
 int32_t skv_probe_read_pages_device(skv_layer *layer, skv_stream stream);
+/* The same launch, each workgroup also writing a split partial of the decode kernel's size
+ * (heads-per-group * head_dim f32, non-temporal stores) into the layer's partial buffer once
+ * its last page has arrived: the least a split-K launch must do before a merge can run. The
+ * layer's partials are overwritten (the next attention call rewrites them anyway). */
+int32_t skv_probe_read_store_pages_device(skv_layer *layer, skv_stream stream);
 /* The merge launch of a decode step at the layer's current length, over whatever split
  * partials the layer's buffers hold (those of its last attention call), into out_dev
  * (q_heads * head_dim f32): behind skv_probe_read_pages_device it is what a decode launch pair

@@ -105,6 +105,7 @@ extern "C" {
     pub fn skv_read_rows_f32(layer: *mut skv_layer, first: usize, n: usize, k_out: *mut f32, v_out: *mut f32) -> i32;
     pub fn skv_gather_device(layer: *mut skv_layer, stream: skv_stream, first: usize, n: usize, k_dst_dev: *mut c_void, v_dst_dev: *mut c_void) -> i32;
     pub fn skv_probe_read_pages_device(layer: *mut skv_layer, stream: skv_stream) -> i32;
+    pub fn skv_probe_read_store_pages_device(layer: *mut skv_layer, stream: skv_stream) -> i32;
     pub fn skv_probe_merge_device(layer: *mut skv_layer, stream: skv_stream, out_dev: *mut f32) -> i32;
     pub fn skv_probe_empty_launch_device(ctx: *mut skv_ctx, stream: skv_stream) -> i32;
     pub fn skv_snapshot_blocks(ctx: *mut skv_ctx, stream: skv_stream, layers: *const *mut skv_layer, n_layers: usize, block_ids: *const usize, n_blocks: usize, out: *mut *mut skv_snapshot) -> i32;

@@ -79,6 +79,7 @@ SIGNATURES = {
     "skv_window_start": (_sz, [_sz, _sz]),
     "skv_resident_capacity": (_i32, [_sz, _sz, _sz, C.POINTER(_sz)]),
     "skv_probe_read_pages_device": (_i32, [_vp, _vp]),
+    "skv_probe_read_store_pages_device": (_i32, [_vp, _vp]),
     "skv_probe_merge_device": (_i32, [_vp, _vp, _vp]),
     "skv_probe_empty_launch_device": (_i32, [_vp, _vp]),
     "skv_f32_to_bf16_bits": (C.c_uint16, [C.c_float]),

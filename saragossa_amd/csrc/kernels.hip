@@ -160,6 +160,14 @@ __global__ __launch_bounds__(512) void probe_read_kernel(ProbeArgs a) {
         }
     }
     if (acc == 0x9e3779b9u && a.sink) a.sink[0] = acc; // keeps the loads alive
+    if (a.part) {
+        // what a split launch has to leave behind: a partial of the decode kernel's size per
+        // workgroup, written after the last page has arrived, with the same non-temporal stores
+        typedef float f32x4_t __attribute__((ext_vector_type(4)));
+        const float x = (float)(acc & 1u);
+        f32x4_t *dst = reinterpret_cast<f32x4_t *>(a.part) + (size_t)(kvh * a.splits + split) * (size_t)(a.part_floats >> 2);
+        for (int u = threadIdx.x; u < (a.part_floats >> 2); u += 512) __builtin_nontemporal_store(f32x4_t{x, x, x, x}, dst + u);
+    }
 }
 
 __global__ __launch_bounds__(512) void probe_empty_kernel(uint32_t *sink) {

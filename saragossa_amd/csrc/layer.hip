@@ -1606,7 +1606,7 @@ int32_t skv_read_rows(skv_layer *L, size_t first, size_t n, uint16_t *k_out, uin
 }
 
 // ---- measurement aids ---------------------------------------------------------------------
-int32_t skv_probe_read_pages_device(skv_layer *L, skv_stream stream) try {
+static int32_t probe_read(skv_layer *L, skv_stream stream, bool store_partials) {
     if (!L) return fail(SKV_ERR_DEVICE, "probe: pointeur nul");
     if (L->len == 0) return fail(SKV_ERR_DIMENSION, "probe: cache vide");
     ProbeArgs a{};
@@ -1616,9 +1616,25 @@ int32_t skv_probe_read_pages_device(skv_layer *L, skv_stream stream) try {
     a.sink = nullptr;
     a.n_pages = (int)std::min<size_t>((L->len + 15) / 16, (size_t)L->n_pages);
     a.splits = (int)std::max<size_t>(std::min<size_t>(decode_target_wgs() / (size_t)L->g.kv_heads, (size_t)a.n_pages), 1);
+    a.splits = std::min(a.splits, L->max_splits);
     a.g = L->g;
+    if (store_partials) {
+        // (o[head_dim] per head of the group, rounded down to whole 16-byte units; m and l are 2 of 258 floats)
+        a.part = L->part_o;
+        a.part_floats = (L->g.gqa * L->g.head_dim) & ~3;
+    }
     SKV_HIP(launch_probe_read(a, as_stream(stream)));
     return SKV_OK;
+}
+
+int32_t skv_probe_read_pages_device(skv_layer *L, skv_stream stream) try {
+    return probe_read(L, stream, false);
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_probe_read_store_pages_device(skv_layer *L, skv_stream stream) try {
+    return probe_read(L, stream, true);
 } catch (...) {
     return skv::fail_exception();
 }

@@ -196,6 +196,8 @@ struct ProbeArgs {
     const uint16_t *v_pool;
     const int32_t *table;
     uint32_t *sink;
+    float *part;     // null = read only; else every workgroup also writes part_floats floats (a multiple of 4)
+    int part_floats;
     int n_pages;
     int splits;
     Geom g;

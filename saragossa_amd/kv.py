@@ -258,6 +258,11 @@ class FullAttentionState:
         decode kernel's grid and access pattern."""
         check(self._l.skv_probe_read_pages_device(self._h, stream))
 
+    def encode_probe_read_store_pages(self, stream) -> None:
+        """The read-only launch plus a split partial of the decode kernel's size written by every
+        workgroup: the least a split-K launch must do."""
+        check(self._l.skv_probe_read_store_pages_device(self._h, stream))
+
     def encode_probe_merge(self, stream, out_ptr) -> None:
         """Measurement aid: the merge launch of a decode step at the current length, over the
         partials the layer's last attention call left."""

@@ -52,6 +52,20 @@ def test_default_run_prints_one_json_line_with_the_agreed_keys():
     assert cb["kind"] == "port" and cb["unit"] == "us/token" and cb["cores"] >= 1 and cb["value"] > 0
     assert d["ceiling"]["read_only_launch_us"] > 0
     assert d["ceiling"]["read_then_merge_launch_pair_us"] >= d["ceiling"]["read_only_launch_us"]
+    assert d["ceiling"]["read_store_then_merge_launch_pair_us"] > 0
+    # the timed kernels produced a context: checked against float64 attention inside the run
+    assert 0 <= d["checked_max_abs"] <= 1e-4
+    # the restore leg carries the reference's state clone beside it
+    assert d["restore"]["cpu_baseline"]["kind"] == "port" and d["restore"]["cpu_baseline"]["value"] > 0
+    # the further legs of the default run: configs[4] at batch 4 and the f32 element
+    legs = d["legs"]
+    for key, dtype in (("configs4_batch4", "bf16"), ("configs2_f32_element", "f32")):
+        leg = legs[key]
+        assert leg["dtype"] == dtype and leg["unit"] == "us/token" and leg["value"] > 0
+        assert 0 <= leg["checked_max_abs"] <= 1e-4
+        lrf = leg["roofline"]
+        assert lrf["bound"] == "hbm" and abs(lrf["frac"] - lrf["achieved"] / lrf["peak"]) < 1e-3
+    assert legs["configs4_batch4"]["config"]["batch"] == 4 and "configs[4]" in legs["configs4_batch4"]["config"]["workload"]
 
 
 @pytest.mark.gpu
