@@ -155,6 +155,16 @@ int32_t skv_ctx_synchronize(skv_ctx *ctx);
  * entry point below serves both; where they differ it says so. */
 int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
                          size_t head_dim, int32_t dtype, size_t window, skv_layer **out);
+/* skv_layer_create with the rollback depth of a ring layer as an argument: the ring keeps
+ * `window` + `rollback_rows` rows (rounded up to whole pages, never more than `capacity`), so a
+ * host whose speculative draft is deeper than the default 32 rows (or that never rolls back:
+ * 0) says so here instead of through the environment. The reference keeps the whole cache and
+ * truncates freely (src/decoder/attention_cache.rs:72-100; rollback in
+ * src/decoder/generation.rs:924-1026); a rollback deeper than the ring kept is reported by
+ * the next attention call. SIZE_MAX = the default (SKV_RING_SLACK_ROWS, else 32); ignored when
+ * `window` is 0. */
+int32_t skv_layer_create_ring(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim,
+                              int32_t dtype, size_t window, size_t rollback_rows, skv_layer **out);
 /* full_attention(capacity, q_heads, kv_heads, head_dim, sampled) (attention.rs:26-45):
  * element type from skv_flag_kv_bf16_for(sampled). */
 int32_t skv_layer_create_for(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
@@ -167,6 +177,9 @@ void skv_layer_destroy(skv_layer *layer);
  * layer takes about half of an f32 one; a ring layer's size follows its window, not capacity. */
 int32_t skv_layer_bytes(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
                         size_t window, uint64_t *bytes);
+/* The same for skv_layer_create_ring (no counterpart in the reference, whose caches are never rings). */
+int32_t skv_layer_bytes_ring(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
+                             size_t window, size_t rollback_rows, uint64_t *bytes);
 /* MemoryGuard::check_allocation (src/memory_guard.rs:365-370) against the context's device:
  * current = device memory in use minus what the context's own arena holds for reuse, limit =
  * device memory - headroom, further capped by static_cap when that is not 0. SKV_ERR_MEMORY

@@ -65,9 +65,11 @@ extern "C" {
     pub fn skv_ctx_destroy(ctx: *mut skv_ctx);
     pub fn skv_ctx_synchronize(ctx: *mut skv_ctx) -> i32;
     pub fn skv_layer_create(ctx: *mut skv_ctx, capacity: usize, q_heads: usize, kv_heads: usize, head_dim: usize, dtype: i32, window: usize, out: *mut *mut skv_layer) -> i32;
+    pub fn skv_layer_create_ring(ctx: *mut skv_ctx, capacity: usize, q_heads: usize, kv_heads: usize, head_dim: usize, dtype: i32, window: usize, rollback_rows: usize, out: *mut *mut skv_layer) -> i32;
     pub fn skv_layer_create_for(ctx: *mut skv_ctx, capacity: usize, q_heads: usize, kv_heads: usize, head_dim: usize, sampled: i32, out: *mut *mut skv_layer) -> i32;
     pub fn skv_layer_destroy(layer: *mut skv_layer);
     pub fn skv_layer_bytes(capacity: usize, q_heads: usize, kv_heads: usize, head_dim: usize, dtype: i32, window: usize, bytes: *mut u64) -> i32;
+    pub fn skv_layer_bytes_ring(capacity: usize, q_heads: usize, kv_heads: usize, head_dim: usize, dtype: i32, window: usize, rollback_rows: usize, bytes: *mut u64) -> i32;
     pub fn skv_check_allocation(ctx: *mut skv_ctx, requested: u64, static_cap: u64, headroom: u64, available: *mut u64, projected: *mut u64) -> i32;
     pub fn skv_layer_set_block_table(layer: *mut skv_layer, table: *const i32, n: usize) -> i32;
     pub fn skv_layer_pages(layer: *const skv_layer) -> usize;

@@ -63,6 +63,7 @@ SIGNATURES = {
     "skv_memory_projection": (_i32, [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64,
                                      C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "skv_layer_bytes": (_i32, [_sz, _sz, _sz, _sz, _i32, _sz, C.POINTER(C.c_uint64)]),
+    "skv_layer_bytes_ring": (_i32, [_sz, _sz, _sz, _sz, _i32, _sz, _sz, C.POINTER(C.c_uint64)]),
     "skv_check_allocation": (_i32, [_vp, C.c_uint64, C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64),
                                     C.POINTER(C.c_uint64)]),
     "skv_decode_step_static_device": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp]),
@@ -87,6 +88,7 @@ SIGNATURES = {
     "skv_ctx_destroy": (None, [_vp]),
     "skv_ctx_synchronize": (_i32, [_vp]),
     "skv_layer_create": (_i32, [_vp, _sz, _sz, _sz, _sz, _i32, _sz, C.POINTER(_vp)]),
+    "skv_layer_create_ring": (_i32, [_vp, _sz, _sz, _sz, _sz, _i32, _sz, _sz, C.POINTER(_vp)]),
     "skv_layer_create_for": (_i32, [_vp, _sz, _sz, _sz, _sz, _i32, C.POINTER(_vp)]),
     "skv_layer_destroy": (None, [_vp]),
     "skv_layer_set_block_table": (_i32, [_vp, _vp, _sz]),

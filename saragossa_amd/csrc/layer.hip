@@ -582,8 +582,10 @@ struct LayerPlan {
     }
 };
 
+// rollback_rows: rows a ring layer keeps behind its window (SIZE_MAX = the default: the
+// environment's SKV_RING_SLACK_ROWS, else 32)
 static int32_t plan_layer(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
-                          size_t window, LayerPlan &p) {
+                          size_t window, size_t rollback_rows, LayerPlan &p) {
     if (capacity == 0 || q_heads == 0 || kv_heads == 0 || head_dim == 0)
         return fail(SKV_ERR_CONFIG, "FullAttentionMetalState: dimension nulle");
     if (q_heads % kv_heads != 0)
@@ -594,7 +596,8 @@ static int32_t plan_layer(size_t capacity, size_t q_heads, size_t kv_heads, size
     const bool f32 = dtype == SKV_DTYPE_F32;
     const int P = padded_head_dim(head_dim);
     if (P == 0) return fail(SKV_ERR_CONFIG, "head_dim > 512 non supporté");
-    if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096 || window > (size_t)1 << 30)
+    if (capacity > (size_t)1 << 30 || q_heads > 4096 || kv_heads > 4096 || window > (size_t)1 << 30 ||
+        (rollback_rows != SIZE_MAX && rollback_rows > (size_t)1 << 30))
         return fail(SKV_ERR_CONFIG, "capacité KV déborde");
     Geom &g = p.g;
     g.q_heads = (int)q_heads;
@@ -612,7 +615,7 @@ static int32_t plan_layer(size_t capacity, size_t q_heads, size_t kv_heads, size
         // what the next query attends: the reference keeps the whole cache and rolls back
         // freely (src/decoder/attention_cache.rs:72-100). A ring never needs more rows than
         // the capacity.
-        const size_t slack = env_usize("SKV_RING_SLACK_ROWS", 32);
+        const size_t slack = rollback_rows != SIZE_MAX ? rollback_rows : env_usize("SKV_RING_SLACK_ROWS", 32);
         size_t ring = (window + slack + 15) / 16 * 16;
         ring = std::min(ring, (capacity + 15) / 16 * 16);
         g.ring_rows = (int)ring;
@@ -634,7 +637,7 @@ int32_t skv_layer_bytes(size_t capacity, size_t q_heads, size_t kv_heads, size_t
                         size_t window, uint64_t *bytes) try {
     if (!bytes) return fail(SKV_ERR_DEVICE, "skv_layer_bytes: pointeur nul");
     LayerPlan p;
-    int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, p);
+    int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, SIZE_MAX, p);
     if (rc) return rc;
     *bytes = (uint64_t)p.total();
     return SKV_OK;
@@ -674,12 +677,29 @@ int32_t skv_check_allocation(skv_ctx *ctx, uint64_t requested, uint64_t static_c
 }
 
 int32_t skv_layer_create(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads,
-                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) try {
+                         size_t head_dim, int32_t dtype, size_t window, skv_layer **out) {
+    return skv_layer_create_ring(ctx, capacity, q_heads, kv_heads, head_dim, dtype, window, SIZE_MAX, out);
+}
+
+int32_t skv_layer_bytes_ring(size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim, int32_t dtype,
+                             size_t window, size_t rollback_rows, uint64_t *bytes) try {
+    if (!bytes) return fail(SKV_ERR_DEVICE, "skv_layer_bytes: pointeur nul");
+    LayerPlan p;
+    int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, rollback_rows, p);
+    if (rc) return rc;
+    *bytes = (uint64_t)p.total();
+    return SKV_OK;
+} catch (...) {
+    return skv::fail_exception();
+}
+
+int32_t skv_layer_create_ring(skv_ctx *ctx, size_t capacity, size_t q_heads, size_t kv_heads, size_t head_dim,
+                              int32_t dtype, size_t window, size_t rollback_rows, skv_layer **out) try {
     if (!ctx || !out) return fail(SKV_ERR_DEVICE, "skv_layer_create: pointeur nul");
     *out = nullptr;
     LayerPlan plan;
     {
-        int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, plan);
+        int32_t rc = plan_layer(capacity, q_heads, kv_heads, head_dim, dtype, window, rollback_rows, plan);
         if (rc) return rc;
     }
     SKV_HIP(hipSetDevice(ctx->device));

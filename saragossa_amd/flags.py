@@ -131,12 +131,16 @@ def memory_projection(current: int, reserved: int, requested: int, limit: int):
     return bool(over), int(proj.value), int(avail.value)
 
 
-def layer_bytes(capacity, q_heads, kv_heads, head_dim, dtype, window=0) -> int:
-    """Device bytes a layer with these arguments takes (skv_layer_bytes)."""
+def layer_bytes(capacity, q_heads, kv_heads, head_dim, dtype, window=0, rollback_rows=None) -> int:
+    """Device bytes a layer with these arguments takes (skv_layer_bytes, skv_layer_bytes_ring)."""
     import ctypes
     from ._lib import check
     out = ctypes.c_uint64(0)
-    check(lib().skv_layer_bytes(capacity, q_heads, kv_heads, head_dim, dtype, window, ctypes.byref(out)))
+    if rollback_rows is None:
+        check(lib().skv_layer_bytes(capacity, q_heads, kv_heads, head_dim, dtype, window, ctypes.byref(out)))
+    else:
+        check(lib().skv_layer_bytes_ring(capacity, q_heads, kv_heads, head_dim, dtype, window, rollback_rows,
+                                         ctypes.byref(out)))
     return int(out.value)
 
 

@@ -43,10 +43,16 @@ class DecodeResidentState:
         check(self._l.skv_ctx_synchronize(self._h))
 
     def full_attention_with_element(self, capacity, q_heads, kv_heads, head_dim,
-                                    dtype=DTYPE_BF16, window=0) -> "FullAttentionState":
+                                    dtype=DTYPE_BF16, window=0, rollback_rows=None) -> "FullAttentionState":
+        """rollback_rows: rows a ring layer (window > 0) keeps behind its window so that a
+        speculative verify of that depth can be rolled back; None = the library's default."""
         h = C.c_void_p()
-        check(self._l.skv_layer_create(self._h, capacity, q_heads, kv_heads, head_dim, dtype,
-                                       window, C.byref(h)))
+        if rollback_rows is None:
+            check(self._l.skv_layer_create(self._h, capacity, q_heads, kv_heads, head_dim, dtype,
+                                           window, C.byref(h)))
+        else:
+            check(self._l.skv_layer_create_ring(self._h, capacity, q_heads, kv_heads, head_dim, dtype,
+                                                window, rollback_rows, C.byref(h)))
         return FullAttentionState(self, h)
 
     def full_attention(self, capacity, q_heads, kv_heads, head_dim, sampled) -> "FullAttentionState":

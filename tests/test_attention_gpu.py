@@ -427,3 +427,71 @@ def test_sdpa_2pass_off_and_min_len(state, env_flags):
         finally:
             os.environ.pop("SKV_DECODE_WGS", None)
         assert np.abs(base - other).max() <= 2e-6
+
+
+@pytest.mark.parametrize("dims,chunk", [((32, 8, 128), 64), ((32, 8, 128), 1000), ((16, 2, 256), 300), ((6, 1, 40), 50),
+                                         ((4, 2, 16), 7)])
+@pytest.mark.parametrize("element", ["bf16", "f32"])
+def test_first_chunk_matches_causal_attention_divide_form(state, dims, chunk, element):
+    """A first chunk from an empty cache is the reference's `causal_attention`
+    (src/decoder/attention_ops.rs:1052-1116): scores are dot / sqrt(attn_scalar), a division,
+    where the cached path multiplies by the reciprocal. The device takes one form for both; it
+    must stay within the bound of either."""
+    q_heads, kv_heads, head_dim = dims
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(chunk * 13 + head_dim)
+    lay = oracle.layout(q_heads, kv_heads, head_dim)
+    q = rng.standard_normal((chunk, q_dim), dtype=np.float32)
+    k = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+    v = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+    make = state.full_attention_bf16 if element == "bf16" else state.full_attention_f32
+    kv = make(chunk, q_heads, kv_heads, head_dim)
+    kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+    got = kv.prefill_rows(q, k, v)
+    # the rows the cache holds (rounded once at the append on a bf16 layer), from the oracle's cache
+    rows = oracle.LayerKvCache("bf16r" if element == "bf16" else "f32")
+    rows.append_batch(k, v, lay)
+    want = oracle.causal_attention(q, rows.keys(), rows.values(), lay)
+    assert np.abs(got - want).max() <= (1e-4 if element == "bf16" else 2e-5), np.abs(got - want).max()
+    kv.close()
+
+
+def test_non_finite_row_in_a_chunk_stays_inside_its_launch_tile(state):
+    """bf16 rounding of a finite f32 at or above 3.39e38 is an infinity (the reference's rounding
+    has no special case, src/decode_resident/utils.rs:55-60), so a live row of a chunk can hold
+    one. The reference's causal loop never reads a later row; a multi-query launch shares each
+    V page among the query slots of a workgroup and masks by the workgroup's range, so there
+    0 x Inf can reach the contexts of earlier query rows of the SAME workgroup tile (at most
+    256 query slots). What is asserted: rows that attend the infinite row are non-finite in
+    both; every row of an earlier workgroup tile equals the oracle's finite context; the
+    infinity is stored as the reference stores it."""
+    q_heads, kv_heads, head_dim = 16, 2, 64
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    start, chunk, bad = 100, 200, 150          # the infinite V row is row `bad` of the chunk
+    rng = np.random.default_rng(77)
+    lay = oracle.layout(q_heads, kv_heads, head_dim)
+    cache = oracle.LayerKvCache("bf16r")
+    kv = state.full_attention_bf16(start + chunk + 4, q_heads, kv_heads, head_dim)
+    k0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+    v0 = rng.standard_normal((start, kv_dim), dtype=np.float32)
+    kv.seed(k0, v0, start)
+    cache.append_batch(k0, v0, lay)
+    q = rng.standard_normal((chunk, q_dim), dtype=np.float32)
+    k = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+    v = rng.standard_normal((chunk, kv_dim), dtype=np.float32)
+    v[bad, 5] = np.float32(3.4e38)             # finite in f32, +Inf once rounded to bf16
+    got = kv.prefill_rows(q, k, v)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle.cached_attention_prefill_rows(q, k, v, cache, lay)
+    gk, gv = kv.read_rows_f32()
+    assert np.array_equal(gk, cache.keys()) and np.array_equal(gv, cache.values())
+    assert np.isinf(gv[start + bad, 5])
+    # rows that attend the infinite row: non-finite in that column of the kv head's query heads, in both
+    gqa = q_heads // kv_heads
+    cols = [h * head_dim + 5 for h in range(gqa)]           # kv head 0 serves query heads 0..gqa-1
+    assert not np.isfinite(want[bad:][:, cols]).any() and not np.isfinite(got[bad:][:, cols]).any()
+    # a workgroup tile holds at most 256 query slots = 256 / gqa rows: rows before that are untouched
+    safe = bad - 256 // gqa
+    assert np.isfinite(got[:safe]).all()
+    assert np.abs(got[:safe] - want[:safe]).max() <= 1e-4
+    kv.close()

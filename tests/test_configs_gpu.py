@@ -25,9 +25,11 @@ def _seed_device(kv, rows, kv_dim, gen):
 
 def test_config2_hybrid_32k_decode_steps(state):
     """configs[2]: full-attention layers 16/2/256 at 32768 cached rows (2 of the 10 identical
-    layers), random block tables, decode steps with fresh q, k, v; the 30 recurrent states
-    (96 KiB conv + 2 MiB ssm each) are snapshotted once and restored byte-identically."""
-    qh, kvh, hd, ctx, steps, n_layers = 16, 2, 256, 32768, 6, 2
+    layers), random block tables, decode steps with fresh q, k, v (20 of them: the cache grows
+    past 32784 rows, so the newest rows start a page the block table has not used yet); the 30
+    recurrent states (96 KiB conv + 2 MiB ssm each) are snapshotted once and restored
+    byte-identically."""
+    qh, kvh, hd, ctx, steps, n_layers = 16, 2, 256, 32768, 20, 2
     kv_dim, q_dim = kvh * hd, qh * hd
     gen = torch.Generator(device="cuda").manual_seed(2)
     rng = np.random.default_rng(2)

@@ -282,3 +282,30 @@ def test_objects_may_outlive_their_context():
         lifetime()
     free1, _ = torch.cuda.mem_get_info()
     assert free0 - free1 <= 16 << 20, (free0, free1)
+
+
+@pytest.mark.parametrize("dtype,window", [(skv.DTYPE_BF16, 0), (skv.DTYPE_F32, 0), (skv.DTYPE_BF16, 1024)])
+def test_layer_bytes_is_what_a_created_layer_takes(dtype, window):
+    """skv_layer_bytes (the figure a host budgets with, as setup.rs:897-962 budgets the resident
+    KV) against the device memory a freshly created layer really takes: a context of its own,
+    so nothing comes out of an arena, and hipMemGetInfo before and after."""
+    torch = pytest.importorskip("torch")
+    from saragossa_amd import flags
+    st = skv.DecodeResidentState(0)
+    try:
+        shape = (65536, 16, 8, 256)
+        torch.cuda.synchronize()
+        free0, _ = torch.cuda.mem_get_info()
+        kv = st.full_attention_with_element(*shape, dtype, window)
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        want = flags.layer_bytes(*shape, dtype, window)
+        took = free0 - free1
+        # the allocator rounds large buffers up to its granule (2 MiB) and carves small ones out of
+        # chunks it already holds, so each of the layer's nine buffers may be off by one granule
+        assert abs(took - want) <= 9 * (2 << 20), (want, took)
+        if want >= 256 << 20:   # where the granules are small against the layer
+            assert 0.98 * took <= want <= 1.02 * took, (want, took)
+        kv.close()
+    finally:
+        st.close()

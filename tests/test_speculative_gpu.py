@@ -70,3 +70,60 @@ def test_rollback_deeper_than_the_rings_slack_is_an_error_not_stale_data(state):
     kv.truncate(101)
     with pytest.raises(skv.DimensionError):
         kv.attention_decode_windowed(q[0], skv.flags.window_start(100, window))
+
+
+@pytest.mark.parametrize("element", ["bf16", "f32"])
+@pytest.mark.parametrize("slack", [0, 16, 64])
+def test_ring_rollback_depth_is_a_create_argument(state, element, slack):
+    """skv_layer_create_ring: a ring layer of window 1024 created with a rollback depth of 0, 16
+    or 64 rows. A verify of up to that many rows can be rolled back completely (the reference
+    truncates freely, src/decoder/attention_cache.rs:72-100; src/decoder/generation.rs:924-1026)
+    and the layer then behaves as if the rows had never been appended; one row more than the
+    depth is reported by the next attention call, never served stale."""
+    q_heads, kv_heads, head_dim, window = 16, 8, 64, 1024
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    rng = np.random.default_rng(1000 + slack)
+    dtype = skv.DTYPE_BF16 if element == "bf16" else skv.DTYPE_F32
+    base = 2 * window + 37                              # the ring has wrapped
+    kv = state.full_attention_with_element(base + 400, q_heads, kv_heads, head_dim, dtype, window, rollback_rows=slack)
+    assert kv.pages() == (window + slack + 15) // 16
+    kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+    assert skv.flags.layer_bytes(base + 400, q_heads, kv_heads, head_dim, dtype, window, rollback_rows=slack) \
+        < skv.flags.layer_bytes(base + 400, q_heads, kv_heads, head_dim, dtype, window, rollback_rows=slack + 4096)
+    lay = oracle.layout(q_heads, kv_heads, head_dim, sliding_window=window)
+    cache = oracle.LayerKvCache("bf16r" if element == "bf16" else "f32")
+    k0 = rng.standard_normal((base, kv_dim), dtype=np.float32)
+    v0 = rng.standard_normal((base, kv_dim), dtype=np.float32)
+    kv.seed(k0, v0, base)
+    cache.append_batch(k0, v0, lay)
+    tol = 1e-4 if element == "bf16" else 2e-5
+    for depth in sorted({1, max(slack, 1)} if slack else {1}):
+        if depth > slack:
+            break
+        q = rng.standard_normal((depth, q_dim), dtype=np.float32)
+        k = rng.standard_normal((depth, kv_dim), dtype=np.float32)
+        v = rng.standard_normal((depth, kv_dim), dtype=np.float32)
+        start = kv.len()
+        kv.prefill_rows(q, k, v)                        # the draft rows
+        kv.truncate(start)                              # all of them rejected
+        qd = rng.standard_normal(q_dim, dtype=np.float32)
+        kd = rng.standard_normal(kv_dim, dtype=np.float32)
+        vd = rng.standard_normal(kv_dim, dtype=np.float32)
+        kv.append_row(kd, vd)
+        got = kv.attention_decode_windowed(qd, skv.flags.window_start(kv.len() - 1, window))
+        want = oracle.decode_step(cache, kd, vd, qd, lay)
+        assert np.abs(got - want).max() <= tol
+    first = kv.len() - window
+    gk, gv = kv.read_rows_f32(first, window)
+    assert np.array_equal(gk, cache.keys()[first:]) and np.array_equal(gv, cache.values()[first:])
+    # one row deeper than the ring kept (the ring holds whole pages, so "kept" is its row count)
+    kept = kv.pages() * 16 - window
+    n_over = kept + 1
+    q = rng.standard_normal((n_over, q_dim), dtype=np.float32)
+    k = rng.standard_normal((n_over, kv_dim), dtype=np.float32)
+    start = kv.len()
+    kv.prefill_rows(q, k, k)
+    kv.truncate(start)
+    with pytest.raises(skv.DimensionError):
+        kv.attention_decode_windowed(q[0], skv.flags.window_start(start - 1, window))
+    kv.close()
