@@ -547,7 +547,10 @@ int32_t skv_prompt_cache_entry(const skv_prompt_cache *cache, size_t index, size
  * (each layer's len must be n_tokens) and of the n_states state buffers, keyed by the prompt's
  * tokens; an entry with the same tokens is replaced, the new entry is the most recent, the
  * least recent ones beyond the capacity are dropped. Async on `stream`; dropping an entry waits
- * for the device before its memory is freed. */
+ * for the device before its memory is freed. Of a ring layer (window > 0) whose prompt is
+ * longer than the ring, the entry holds the pages the ring still holds (the reference clones
+ * the whole cache, but its sliding layers never attend the older rows again); a hit restores
+ * them into ring layers only, with the oldest kept row as the layer's floor. */
 int32_t skv_prompt_cache_put(skv_prompt_cache *cache, skv_stream stream, const uint64_t *tokens,
                              size_t n_tokens, skv_layer *const *layers, size_t n_layers,
                              const void *const *state_ptrs, const size_t *state_bytes, size_t n_states);

@@ -874,6 +874,10 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
 
 struct PromptEntry {
     std::vector<uint64_t> tokens;
+    // per layer: logical pages below this one are not in the snapshot (a ring layer whose
+    // prompt was longer than the ring no longer held them; the reference clones the whole
+    // cache, generation.rs:3105-3139, but its sliding layers never attend those rows again)
+    std::vector<uint32_t> first_page;
     skv_snapshot *pages = nullptr;
     skv_snapshot *state = nullptr;
     size_t bytes = 0;
@@ -968,10 +972,38 @@ int32_t skv_prompt_cache_put(skv_prompt_cache *c, skv_stream stream, const uint6
     // the snapshots first: a failure leaves the cache as it was
     PromptEntry e;
     e.tokens.assign(tokens, tokens + n_tokens);
-    std::vector<size_t> blocks((n_tokens + 15) / 16);
-    for (size_t i = 0; i < blocks.size(); ++i) blocks[i] = i;
-    rc = skv_snapshot_blocks(c->ctx, stream, layers, n_layers, blocks.data(), blocks.size(), &e.pages);
-    if (rc) return rc;
+    const size_t n_blocks = (n_tokens + 15) / 16;
+    // a ring layer holds positions floor_pos .. len-1: its whole pages from the first one that
+    // starts at or after floor_pos (the page that straddles floor_pos already holds newer rows
+    // in its low slots; its surviving rows lie behind every window the layer can still serve
+    // as long as the ring keeps 16 rows or more behind the window)
+    e.first_page.assign(n_layers, 0);
+    for (size_t l = 0; l < n_layers; ++l)
+        if (layers[l]->g.ring_rows > 0) e.first_page[l] = (uint32_t)((layers[l]->floor_pos + 15) / 16);
+    {
+        SKV_HIP(hipSetDevice(c->ctx->device));
+        skv_snapshot *snap = new skv_snapshot();
+        snap->ctx = c->ctx;
+        snap->layout.build(layers, n_layers);
+        snap->n_pages = n_blocks;
+        snap->bytes = n_blocks * snap->layout.slot_bytes;
+        if (snap->bytes) {
+            hipError_t he = hipMalloc((void **)&snap->base, snap->bytes);
+            if (he != hipSuccess) {
+                delete snap;
+                return fail_hip(he, "prompt_cache_put: allocation");
+            }
+            std::vector<int32_t> pages(n_blocks), slots(n_blocks);
+            for (size_t i = 0; i < n_blocks; ++i) pages[i] = slots[i] = (int32_t)i;
+            rc = copy_pages(snap->layout, snap->base, layers, n_layers, pages.data(), slots.data(), n_blocks,
+                            e.first_page.data(), true, as_stream(stream));
+            if (rc) {
+                skv_snapshot_free(snap);
+                return rc;
+            }
+        }
+        e.pages = snap;
+    }
     rc = skv_state_snapshot(c->ctx, stream, state_ptrs, state_bytes, n_states, &e.state);
     if (rc) {
         prompt_entry_free(e);
@@ -1017,15 +1049,37 @@ int32_t skv_prompt_cache_get(skv_prompt_cache *c, skv_stream stream, const uint6
     for (size_t i = 0; i < n_states; ++i)
         if (!state_ptrs || !state_bytes || state_bytes[i] != hit.state->sizes[i])
             return fail(SKV_ERR_DIMENSION, "prompt_cache_get: taille du tampon d'état " + std::to_string(i) + " différente");
-    std::vector<size_t> blocks(hit.pages ? hit.pages->n_pages : 0);
-    for (size_t i = 0; i < blocks.size(); ++i) blocks[i] = i;
-    rc = skv_restore_blocks(c->ctx, stream, hit.pages, layers, n_layers, blocks.data(), blocks.size());
-    if (rc) return rc;
+    const size_t n_blocks = hit.pages ? hit.pages->n_pages : 0;
+    if (n_blocks && (hit.first_page.size() != n_layers || !hit.pages->layout.matches(layers, n_layers)))
+        return fail(SKV_ERR_DIMENSION, "prefix-cache: snapshots=" + std::to_string(hit.first_page.size()) +
+                                           " couches=" + std::to_string(n_layers) + " ou formes différentes");
+    // where each layer's restored pages start: what the entry holds, and no more than the
+    // destination's own ring can take
+    std::vector<uint32_t> first_page(n_layers, 0);
+    for (size_t l = 0; l < n_layers && n_blocks; ++l) {
+        const skv_layer *L = layers[l];
+        first_page[l] = hit.first_page[l];
+        if (L->g.ring_rows == 0) {
+            if (first_page[l] > 0)
+                return fail(SKV_ERR_DIMENSION, "prompt_cache_get: l'entrée ne tient que la fenêtre de la couche " +
+                                                   std::to_string(l) + ", la couche de destination n'est pas un anneau");
+        } else if (cached > (size_t)L->g.ring_rows) {
+            first_page[l] = std::max(first_page[l], (uint32_t)((cached - (size_t)L->g.ring_rows + 15) / 16));
+        }
+    }
+    if (n_blocks) {
+        SKV_HIP(hipSetDevice(c->ctx->device));
+        std::vector<int32_t> pages(n_blocks), slots(n_blocks);
+        for (size_t i = 0; i < n_blocks; ++i) pages[i] = slots[i] = (int32_t)i;
+        rc = copy_pages(hit.pages->layout, hit.pages->base, layers, n_layers, pages.data(), slots.data(), n_blocks,
+                        first_page.data(), false, as_stream(stream));
+        if (rc) return rc;
+    }
     rc = skv_state_restore(c->ctx, stream, hit.state, state_ptrs, state_bytes, n_states);
     if (rc) return rc;
     for (size_t l = 0; l < n_layers; ++l) {
         layers[l]->len = cached;
-        layers[l]->floor_pos = 0;
+        layers[l]->floor_pos = (size_t)first_page[l] * 16;
     }
     // the hit becomes the most recent entry (generation.rs:3007-3012)
     if (index > 0) std::rotate(c->entries.begin(), c->entries.begin() + index, c->entries.begin() + index + 1);

@@ -452,3 +452,71 @@ def test_whole_prompt_cache_follows_the_reference(state, element):
     assert len(off) == 0 and off.lookup(top, layers, ptrs, sizes) == 0
     off.close()
     cache.close()
+
+
+@pytest.mark.parametrize("n_prompt", [40, 96, 300, 1000])
+def test_whole_prompt_cache_with_sliding_window_layers(state, element, n_prompt):
+    """The whole-prompt cache over a model with sliding-window layers (ring buffers): a prompt
+    shorter than the ring, one that just fills it and ones that wrapped it several times. The
+    reference's put clones the whole cache whatever the window (generation.rs:3105-3139); its
+    sliding layers never attend rows behind the window again, so here an entry holds a ring
+    layer's live pages only. After a hit the full layer holds every row, the ring layers the
+    last `window` rows, bit for bit, and decode steps on all of them equal the oracle's."""
+    dims, window = (8, 2, 64), 64
+    kv_dim, q_dim = dims[1] * dims[2], dims[0] * dims[2]
+    rng = np.random.default_rng(n_prompt)
+    prompt = [int(t) for t in rng.integers(0, 151936, size=n_prompt)]
+    tail = [int(t) for t in rng.integers(0, 151936, size=23)]
+    windows = [0, window, window]
+    make = state.full_attention_f32 if ELEMENT == "f32" else state.full_attention_bf16
+
+    def build():
+        out = []
+        for li, w in enumerate(windows):
+            kv = make(n_prompt + 64, *dims, window=w)
+            kv.set_block_table(np.random.default_rng(li + n_prompt).permutation(kv.pages()).astype(np.int32))
+            out.append(kv)
+        return out
+
+    cache = skv.WholePromptCache(state, capacity=2)
+    src = build()
+    fill(src, 0, n_prompt, prompt, kv_dim)
+    cache.put(prompt, src, stream=_stream())
+    dst = build()
+    assert cache.lookup(prompt + tail, dst, stream=_stream()) == n_prompt
+    torch.cuda.synchronize()
+    fill(dst, n_prompt, n_prompt + len(tail), prompt + tail, kv_dim)     # the request goes on from the hit
+    n = n_prompt + len(tail)
+    mode = "f32" if ELEMENT == "f32" else "bf16r"
+    for li, (kv, w) in enumerate(zip(dst, windows)):
+        assert kv.len() == n
+        first = 0 if w == 0 else max(0, n - w)
+        k, v = rows_for(li, range(n), prompt + tail, kv_dim)
+        lay = oracle.layout(*dims, sliding_window=w)
+        c = oracle.LayerKvCache(mode)
+        c.append_batch(k, v, lay)
+        gk, gv = kv.read_rows_f32(first, n - first)
+        assert np.array_equal(gk, c.keys()[first:]) and np.array_equal(gv, c.values()[first:]), li
+        q = rng.standard_normal(q_dim, dtype=np.float32)
+        got = kv.attention_decode_windowed(q, skv.flags.window_start(n - 1, w))
+        assert np.abs(got - oracle.cached_attention_one(q, c, lay)).max() <= 1e-4, li
+    # the entry is untouched by what the request appended: a second hit restores the same rows
+    again = build()
+    assert cache.lookup(prompt, again, stream=_stream()) == n_prompt
+    torch.cuda.synchronize()
+    k, v = rows_for(1, range(n_prompt), prompt, kv_dim)
+    first = max(0, n_prompt - window)
+    c = oracle.LayerKvCache(mode)
+    c.append_batch(k, v, oracle.layout(*dims, sliding_window=window))
+    gk, gv = again[1].read_rows_f32(first, n_prompt - first)
+    assert np.array_equal(gk, c.keys()[first:]) and np.array_equal(gv, c.values()[first:])
+    # an entry that holds only a ring layer's window cannot fill a layer that keeps every row
+    if n_prompt > window + 48:
+        full = [make(n_prompt + 64, *dims) for _ in windows]
+        with pytest.raises(skv.DimensionError):
+            cache.lookup(prompt, full, stream=_stream())
+        assert all(kv.len() == 0 for kv in full)
+        for kv in full:
+            kv.close()
+    for kv in src + dst + again:
+        kv.close()
