@@ -17,8 +17,20 @@ struct skv_ctx {
     void *static_scratch = nullptr; // this device's copy of the library's static scratch array
     // Split-K partials of multi-query launches (chunked prefill), one buffer per stream the
     // context has seen such a launch on, grown on demand: launches on one stream are ordered by
-    // it, launches on different streams never share a buffer. Guarded by arena_mu.
-    std::map<hipStream_t, std::pair<void *, size_t>> mq_scratch;
+    // it, launches on different streams never share a buffer. At most MQ_SCRATCH_STREAMS
+    // entries: a caller that makes a stream per request would otherwise leave one buffer per
+    // dead stream behind; past that the least recently used entry is dropped (after a device
+    // synchronisation: its stream may no longer exist). The map is guarded by arena_mu; the
+    // waits, frees and allocations happen outside it. Calls on ONE stream must come from one
+    // thread at a time (as a stream's owner issues its work anyway).
+    struct MqScratch {
+        void *ptr = nullptr;
+        size_t bytes = 0;
+        uint64_t used = 0; // value of mq_clock at the last use
+    };
+    static constexpr size_t MQ_SCRATCH_STREAMS = 8;
+    std::map<hipStream_t, MqScratch> mq_scratch;
+    uint64_t mq_clock = 0;
     // Device buffers of destroyed layers, kept for the next layer that needs about as much:
     // the stand-in for the arena DecodeResidentState leases its buffers from
     // (src/decode_resident/arena.rs:116-211). A server creates and drops one cache per layer

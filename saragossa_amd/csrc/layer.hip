@@ -65,7 +65,7 @@ void arena_put(skv_ctx *ctx, void *ptr, size_t bytes) {
 static void ctx_drain(skv_ctx *ctx) {
     std::lock_guard<std::mutex> lk(ctx->arena_mu);
     for (auto &kv : ctx->mq_scratch)
-        if (kv.second.first) (void)hipFree(kv.second.first);
+        if (kv.second.ptr) (void)hipFree(kv.second.ptr);
     ctx->mq_scratch.clear();
     for (auto &kv : ctx->arena_free) (void)hipFree(kv.second);
     ctx->arena_free.clear();
@@ -278,19 +278,44 @@ int32_t multi_query_partials(skv_layer *L, hipStream_t s, size_t n_sets, size_t 
     const size_t need = n_part * ((size_t)g.head_dim + 2) * sizeof(float);
     skv_ctx *c = L->ctx;
     void *buf = nullptr;
+    void *old = nullptr;     // this stream's buffer, too small: freed once the stream has drained
+    void *evicted = nullptr; // another stream's buffer, pushed out of the bounded map
     {
         std::lock_guard<std::mutex> lk(c->arena_mu);
-        auto &slot = c->mq_scratch[s];
-        if (slot.second < need) {
-            // work queued on the stream may still read the old buffer
-            SKV_HIP(hipStreamSynchronize(s));
-            if (slot.first) SKV_HIP(hipFree(slot.first));
-            slot = {nullptr, 0};
-            void *p = nullptr;
-            SKV_HIP(hipMalloc(&p, need));
-            slot = {p, need};
+        auto it = c->mq_scratch.find(s);
+        if (it != c->mq_scratch.end() && it->second.bytes >= need) {
+            it->second.used = ++c->mq_clock;
+            buf = it->second.ptr;
+        } else if (it != c->mq_scratch.end()) {
+            old = it->second.ptr;
+            c->mq_scratch.erase(it); // nobody else uses this stream's entry (one thread per stream)
+        } else if (c->mq_scratch.size() >= skv_ctx::MQ_SCRATCH_STREAMS) {
+            auto lru = c->mq_scratch.begin();
+            for (auto j = c->mq_scratch.begin(); j != c->mq_scratch.end(); ++j)
+                if (j->second.used < lru->second.used) lru = j;
+            evicted = lru->second.ptr;
+            c->mq_scratch.erase(lru);
         }
-        buf = slot.first;
+    }
+    if (!buf) {
+        // waits, frees and the allocation outside the lock: other threads' arena_get / arena_put
+        // and launches on other streams go on meanwhile
+        if (old) {
+            SKV_HIP(hipStreamSynchronize(s)); // work queued on the stream may still read it
+            SKV_HIP(hipFree(old));
+        }
+        if (evicted) {
+            SKV_HIP(hipDeviceSynchronize()); // its stream may be gone: wait for everything
+            SKV_HIP(hipFree(evicted));
+        }
+        void *p = nullptr;
+        SKV_HIP(hipMalloc(&p, need));
+        std::lock_guard<std::mutex> lk(c->arena_mu);
+        skv_ctx::MqScratch &slot = c->mq_scratch[s];
+        slot.ptr = p;
+        slot.bytes = need;
+        slot.used = ++c->mq_clock;
+        buf = p;
     }
     a.part_o = reinterpret_cast<float *>(buf);
     a.part_m = a.part_o + n_part * g.head_dim;

@@ -107,3 +107,53 @@ def test_static_scratch_step_rejects_what_does_not_fit(state):
         kv.encode_decode_step_static(_stream(), z.data_ptr(), 0, z.data_ptr(), 0, q.data_ptr(), out.data_ptr())
     assert kv.len() == rows
     torch.cuda.synchronize()
+
+
+def test_static_scratch_step_on_wide_f32_heads_takes_the_separate_launches(state):
+    """f32 rows of head_dim 512 have no fused append: the entry point appends, then attends with
+    the partials in the static array (its other branch)."""
+    dims = (16, 8, 512)
+    layers, cache, lay, rng = _pair(state, dims, 2000, 0, skv.DTYPE_F32, 25)
+    _steps(layers, cache, lay, rng, dims, 3)
+
+
+@pytest.mark.parametrize("dtype", [skv.DTYPE_BF16, skv.DTYPE_F32])
+def test_static_scratch_step_is_captured_into_a_graph_and_replayed(state, dtype):
+    """What the entry point exists for: a caller under HIP graph capture, where an allocation, a
+    free or a synchronisation fails the capture. One call is captured (after an eager call, so
+    that per-kernel set-up is done), the graph replayed three times with a new query each time
+    and eager work in between; every replay's context equals the plain attention call of a twin
+    layer over the same rows. (A replay re-runs the captured launch: the same row is written
+    to the same slot again and the same length is attended.)"""
+    dims = (16, 2, 256)
+    q_heads, kv_heads, head_dim = dims
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    layers, cache, lay, rng = _pair(state, dims, 5000, 0, dtype, 26)
+    _steps(layers, cache, lay, rng, dims, 1)                 # eager first: kernels loaded, attributes set
+    static, plain = layers
+    kd = _dev(rng.standard_normal(kv_dim, dtype=np.float32))
+    vd = _dev(rng.standard_normal(kv_dim, dtype=np.float32))
+    qd = _dev(rng.standard_normal(q_dim, dtype=np.float32))
+    out_s = torch.zeros(q_dim, device="cuda", dtype=torch.float32)
+    out_p = torch.zeros(q_dim, device="cuda", dtype=torch.float32)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static.encode_decode_step_static(torch.cuda.current_stream().cuda_stream, kd.data_ptr(), 0, vd.data_ptr(), 0,
+                                         qd.data_ptr(), out_s.data_ptr())
+    assert static.len() == plain.len() + 1                  # the bookkeeping advanced at capture time
+    plain.encode_append_kv(_stream(), kd.data_ptr(), vd.data_ptr())
+    for r in range(3):
+        qd.copy_(_dev(rng.standard_normal(q_dim, dtype=np.float32)))
+        out_s.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        plain.encode_attention_decode_windowed(_stream(), qd.data_ptr(), out_p.data_ptr(), 0)
+        torch.cuda.synchronize()
+        assert np.array_equal(out_s.cpu().numpy(), out_p.cpu().numpy()), r
+        # the program's own eager work between the replays
+        scratch = torch.randn(1 << 20, device="cuda")
+        assert float(scratch.abs().sum()) > 0
+    sk, sv = static.read_rows_f32(static.len() - 8, 8)
+    pk, pv = plain.read_rows_f32(plain.len() - 8, 8)
+    assert np.array_equal(sk, pk) and np.array_equal(sv, pv)
