@@ -277,18 +277,43 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
             sb0[t] = float4_t{0.f, 0.f, 0.f, 0.f};
             sb1[t] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
+        // The operands of a K-step are asked for DEPTH K-steps before its products are issued,
+        // and the order is pinned: left to itself the compiler keeps one read ahead, issues the
+        // product that needs the newest operand first, and every other product then waits for
+        // LDS (the two wavefronts of a SIMD cannot cover a latency each of them hits at once).
+        constexpr int DEPTH = (KK < 2 || P > 256) ? 1 : 2;
+        uint4 ra[KK], rb[KK];
+#pragma unroll
+        for (int kk = 0; kk < DEPTH; ++kk) {
+            ra[kk] = kt_a[kk * 64 + lane];
+            rb[kk] = kt_b[kk * 64 + lane];
+        }
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-            const bf16x8_t ka = __builtin_bit_cast(bf16x8_t, kt_a[kk * 64 + lane]);
-            const bf16x8_t kb = __builtin_bit_cast(bf16x8_t, kt_b[kk * 64 + lane]);
+            if (kk + DEPTH < KK) {
+                ra[kk + DEPTH] = kt_a[(kk + DEPTH) * 64 + lane];
+                rb[kk + DEPTH] = kt_b[(kk + DEPTH) * 64 + lane];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const bf16x8_t ka = __builtin_bit_cast(bf16x8_t, ra[kk]);
+            const bf16x8_t kb = __builtin_bit_cast(bf16x8_t, rb[kk]);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 sa0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qh[t][kk], sa0[t], 0, 0, 0);
-                sa1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, ql[t][kk], sa1[t], 0, 0, 0);
                 sb0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qh[t][kk], sb0[t], 0, 0, 0);
+                sa1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, ql[t][kk], sa1[t], 0, 0, 0);
                 sb1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, ql[t][kk], sb1[t], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        // the first V operands of the pair travel while the softmax runs
+        uint4 rv0[KK], rv1[KK];
+#pragma unroll
+        for (int kk = 0; kk < DEPTH; ++kk) {
+            rv0[kk] = vt[kk * 128 + lane];
+            rv1[kk] = vt[kk * 128 + 64 + lane];
+        }
+        __builtin_amdgcn_sched_barrier(0);
         bf16x8_t ph[TILES], pl[TILES];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
@@ -348,10 +373,16 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
         // O^T += V^T . P^T over the 32 keys of the pair, the V registers shared by the tiles.
         // Without a page B its probabilities are zero and its place holds a page the layer
         // owns (fetch_step clamps), so the products vanish.
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-            const bf16x8_t v0 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + lane]);
-            const bf16x8_t v1 = __builtin_bit_cast(bf16x8_t, vt[kk * 128 + 64 + lane]);
+            if (kk + DEPTH < KK) {
+                rv0[kk + DEPTH] = vt[(kk + DEPTH) * 128 + lane];
+                rv1[kk + DEPTH] = vt[(kk + DEPTH) * 128 + 64 + lane];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const bf16x8_t v0 = __builtin_bit_cast(bf16x8_t, rv0[kk]);
+            const bf16x8_t v1 = __builtin_bit_cast(bf16x8_t, rv1[kk]);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 o[t][2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, ph[t], o[t][2 * kk], 0, 0, 0);
@@ -359,6 +390,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
                 o[t][2 * kk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, pl[t], o[t][2 * kk], 0, 0, 0);
                 o[t][2 * kk + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, pl[t], o[t][2 * kk + 1], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
       }
       store_step<P, PG, THREADS>(stage, kv_lds + ((step + 1) & 1) * BUF_U4, tid, a, pb0, min(step + 1, n_steps - 1),
