@@ -201,6 +201,55 @@ def bench_restore(skv, torch, np, state, stream, element="bf16"):
     return out
 
 
+def bench_sdpa_sweep(skv, torch, np, state, stream, iters=100):
+    """The reference's own SDPA micro-benchmark (attention_decode_bench,
+    src/decode_resident/tests.rs:1494-1541): decode attention alone at q16/kv2/hd256 over 1024,
+    4096, 16384 and 32768 cached rows of its arithmetic test data, ms per call and effective GB/s
+    over the K and V bytes read once. The reference times its synchronous host call on an f32
+    cache (greedy policy); here each length is timed on both elements, as device launches back
+    to back (HIP events) and, like the reference, as the synchronous host call (query in, context
+    out over PCIe, a stream synchronisation per call)."""
+    qh, kvh, hd = 16, 2, 256
+    kv_dim, q_dim = kvh * hd, qh * hd
+    dev = torch.device("cuda:0")
+    q_host = ((np.arange(q_dim) % 89).astype(np.float32) - 44.0) * np.float32(0.01)
+    q = torch.from_numpy(q_host).to(dev)
+    out = torch.empty(q_dim, device=dev, dtype=torch.float32)
+    rows = []
+    for n in (1024, 4096, 16384, 32768):
+        idx = torch.arange(n * kv_dim, device=dev, dtype=torch.int64)
+        k = (((idx % 101).to(torch.float32) - 50.0) * 0.01).view(n, kv_dim)
+        v = (((idx % 97).to(torch.float32) - 48.0) * 0.01).view(n, kv_dim)
+        for element, esize in (("f32", 4), ("bf16", 2)):
+            kv = (state.full_attention_f32 if element == "f32" else state.full_attention_bf16)(n, qh, kvh, hd)
+            kv.encode_append_batch(stream, k.data_ptr(), v.data_ptr(), n)
+            for _ in range(5):
+                kv.encode_attention_decode(stream, q.data_ptr(), out.data_ptr())
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(iters):
+                kv.encode_attention_decode(stream, q.data_ptr(), out.data_ptr())
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / iters
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                kv.attention_decode(q_host)
+            host_ms = (time.perf_counter() - t0) * 1e3 / iters
+            nbytes = n * kv_dim * esize * 2
+            rows.append({"len": n, "element": element, "us_per_call": round(us, 2),
+                         "gbps_effective": round(nbytes / us / 1e3, 1),
+                         "host_call_ms_per_call": round(host_ms, 4),
+                         "host_call_gbps_effective": round(nbytes / host_ms / 1e6, 1)})
+            kv.close()
+        del idx, k, v
+    return {"workload": "attention_decode_bench of the reference (src/decode_resident/tests.rs:1494-1541): "
+                        "q16/kv2/hd256, decode attention alone, %d calls per length" % iters,
+            "rows": rows}
+
+
 def bench_prefill(skv, torch, np, state, stream, element="bf16"):
     """Chunked prefill over the cache (cached_attention_prefill_rows as one launch): a
     512-row chunk appended and attended causally over the rows already cached, at the KV
@@ -968,6 +1017,7 @@ def decode_bench(args, skv, torch, np, state, main_leg):
         result["end_to_end"] = bench_end_to_end(skv, torch, np, state)
     if args.config == 2 and not no_restore:
         result["prefill"] = bench_prefill(skv, torch, np, state, stream, args.element)
+        result["sdpa_sweep"] = bench_sdpa_sweep(skv, torch, np, state, stream)
 
     if not no_cpu:
         import oracle

@@ -102,6 +102,16 @@ size_t skv_flag_serve_prefix_blocks_per_session(void); /* runtime_flags.rs:750-7
 int32_t skv_flag_prefix_cache_enabled(void);      /* RETI_RUST_PREFIX_CACHE, runtime_flags.rs:665-668 */
 size_t skv_flag_prefix_cache_capacity(void);      /* RETI_RUST_PREFIX_CACHE_CAP, runtime_flags.rs:670-678 */
 size_t skv_flag_prefill_chunk(void);              /* RETI_RUST_PREFILL_CHUNK (alias _STEP_SIZE), runtime_flags.rs:414-423 */
+/* The switches and limits of the memory guard that drives prefix-block eviction
+ * (src/serve/state.rs:226-238, 287-306, 627-635): a host feeds them to skv_check_allocation /
+ * skv_memory_projection. A cap of 0 = none set (the reference's None; a zero in the
+ * environment is filtered out). */
+int32_t skv_flag_memory_guard_enabled(void);          /* RETI_MEMORY_GUARD, runtime_flags.rs:699-702 */
+int32_t skv_flag_serve_oom_guard_enabled(void);       /* memory guard && RETI_SERVE_OOM_GUARD, runtime_flags.rs:693-696 */
+uint64_t skv_flag_memory_static_cap_bytes(void);      /* RETI_MEMORY_CAP_BYTES, runtime_flags.rs:705-713 */
+uint64_t skv_flag_memory_headroom_bytes(void);        /* RETI_MEMORY_HEADROOM_BYTES, default 2 GiB, runtime_flags.rs:716-724 */
+uint64_t skv_flag_serve_memory_static_cap_bytes(void);   /* RETI_SERVE_MEMORY_CAP_BYTES, runtime_flags.rs:773-781 */
+uint64_t skv_flag_serve_memory_headroom_bytes(void);     /* RETI_SERVE_MEMORY_HEADROOM_BYTES, default 2 GiB, runtime_flags.rs:784-792 */
 /* The reference freezes each flag at first read (OnceLock). This re-reads the
  * environment; it exists for tests only. */
 void skv_flags_reload(void);

@@ -55,6 +55,12 @@ extern "C" {
     pub fn skv_flag_prefix_cache_enabled() -> i32;
     pub fn skv_flag_prefix_cache_capacity() -> usize;
     pub fn skv_flag_prefill_chunk() -> usize;
+    pub fn skv_flag_memory_guard_enabled() -> i32;
+    pub fn skv_flag_serve_oom_guard_enabled() -> i32;
+    pub fn skv_flag_memory_static_cap_bytes() -> u64;
+    pub fn skv_flag_memory_headroom_bytes() -> u64;
+    pub fn skv_flag_serve_memory_static_cap_bytes() -> u64;
+    pub fn skv_flag_serve_memory_headroom_bytes() -> u64;
     pub fn skv_flags_reload();
     pub fn skv_window_start(position: usize, window: usize) -> usize;
     pub fn skv_resident_capacity(prefill_len: usize, max_new_tokens: usize, draft_headroom: usize, capacity: *mut usize) -> i32;

@@ -76,6 +76,12 @@ SIGNATURES = {
     "skv_flag_prefix_cache_enabled": (_i32, []),
     "skv_flag_prefix_cache_capacity": (_sz, []),
     "skv_flag_prefill_chunk": (_sz, []),
+    "skv_flag_memory_guard_enabled": (_i32, []),
+    "skv_flag_serve_oom_guard_enabled": (_i32, []),
+    "skv_flag_memory_static_cap_bytes": (C.c_uint64, []),
+    "skv_flag_memory_headroom_bytes": (C.c_uint64, []),
+    "skv_flag_serve_memory_static_cap_bytes": (C.c_uint64, []),
+    "skv_flag_serve_memory_headroom_bytes": (C.c_uint64, []),
     "skv_flags_reload": (None, []),
     "skv_window_start": (_sz, [_sz, _sz]),
     "skv_resident_capacity": (_i32, [_sz, _sz, _sz, C.POINTER(_sz)]),

@@ -76,9 +76,17 @@ template <typename T> struct Once {
     }
 };
 
-Once<int> f_flash, f_2pass, f_res_full, f_res, f_serve_prefix, f_prefix, f_kv_bf16, f_sim_k, f_sim_v, f_pipeline;
+Once<int> f_flash, f_2pass, f_res_full, f_res, f_serve_prefix, f_prefix, f_kv_bf16, f_sim_k, f_sim_v, f_pipeline,
+    f_mem_guard, f_oom_guard;
 Once<size_t> f_2pass_min, f_block_tokens, f_cache_blocks, f_per_session, f_prefix_cap, f_chunk, f_par_threshold,
     f_split_min;
+Once<uint64_t> f_mem_cap, f_mem_headroom, f_serve_cap, f_serve_headroom;
+
+// `.ok().and_then(|value| value.trim().parse::<u64>().ok())`
+std::optional<uint64_t> env_u64(const char *name) {
+    auto v = parse_usize(std::getenv(name), true);
+    return v.has_value() ? std::optional<uint64_t>((uint64_t)*v) : std::nullopt;
+}
 
 } // namespace
 
@@ -174,6 +182,28 @@ int32_t skv_flag_prefix_cache_enabled(void) {
 size_t skv_flag_prefix_cache_capacity(void) {
     return f_prefix_cap.get(
         [] { return parse_usize(std::getenv("RETI_RUST_PREFIX_CACHE_CAP"), true).value_or(4); });
+}
+int32_t skv_flag_memory_guard_enabled(void) {
+    return f_mem_guard.get([] { return (int)env_flag("RETI_MEMORY_GUARD", true); });
+}
+int32_t skv_flag_serve_oom_guard_enabled(void) {
+    // memory_guard_enabled() && env_flag("RETI_SERVE_OOM_GUARD", true)
+    const int guard = skv_flag_memory_guard_enabled();
+    return f_oom_guard.get([guard] { return (int)(guard && env_flag("RETI_SERVE_OOM_GUARD", true)); });
+}
+uint64_t skv_flag_memory_static_cap_bytes(void) {
+    // Option<u64> with zero filtered out: 0 = no cap
+    return f_mem_cap.get([] { return env_u64("RETI_MEMORY_CAP_BYTES").value_or(0); });
+}
+uint64_t skv_flag_memory_headroom_bytes(void) {
+    return f_mem_headroom.get([] { return env_u64("RETI_MEMORY_HEADROOM_BYTES").value_or(2ull * 1024 * 1024 * 1024); });
+}
+uint64_t skv_flag_serve_memory_static_cap_bytes(void) {
+    return f_serve_cap.get([] { return env_u64("RETI_SERVE_MEMORY_CAP_BYTES").value_or(0); });
+}
+uint64_t skv_flag_serve_memory_headroom_bytes(void) {
+    return f_serve_headroom.get(
+        [] { return env_u64("RETI_SERVE_MEMORY_HEADROOM_BYTES").value_or(2ull * 1024 * 1024 * 1024); });
 }
 size_t skv_flag_prefill_chunk(void) {
     return f_chunk.get([] {

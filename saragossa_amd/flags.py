@@ -93,6 +93,34 @@ def prefill_chunk_size() -> int:
     return lib().skv_flag_prefill_chunk()
 
 
+def memory_guard_enabled() -> bool:
+    """memory_guard_enabled (src/runtime_flags.rs:699-702)."""
+    return bool(lib().skv_flag_memory_guard_enabled())
+
+
+def serve_oom_guard_enabled() -> bool:
+    """serve_oom_guard_enabled (src/runtime_flags.rs:693-696)."""
+    return bool(lib().skv_flag_serve_oom_guard_enabled())
+
+
+def memory_static_cap_bytes():
+    """memory_static_cap_bytes (src/runtime_flags.rs:705-713): None when unset, unparsable or zero."""
+    return lib().skv_flag_memory_static_cap_bytes() or None
+
+
+def memory_headroom_bytes() -> int:
+    return lib().skv_flag_memory_headroom_bytes()
+
+
+def serve_memory_static_cap_bytes():
+    """serve_memory_static_cap_bytes (src/runtime_flags.rs:773-781)."""
+    return lib().skv_flag_serve_memory_static_cap_bytes() or None
+
+
+def serve_memory_headroom_bytes() -> int:
+    return lib().skv_flag_serve_memory_headroom_bytes()
+
+
 def reload() -> None:
     """Re-read the environment (the reference freezes flags at first read). Tests only."""
     lib().skv_flags_reload()

@@ -73,7 +73,10 @@ def _flags_in_subprocess(env):
             "blocks=f.serve_prefix_cache_blocks(), per=f.serve_prefix_blocks_per_session(),"
             "pc=f.prefix_cache_enabled(), cap=f.prefix_cache_capacity(), chunk=f.prefill_chunk_size(),"
             "split=f.effective_split_min_len(), simk=f.kv_bf16_sim_konly(), simv=f.kv_bf16_sim_vonly(),"
-            "par=f.attention_parallel_threshold(), pipe=f.decode_pipeline_enabled())))")
+            "par=f.attention_parallel_threshold(), pipe=f.decode_pipeline_enabled(),"
+            "guard=f.memory_guard_enabled(), oom=f.serve_oom_guard_enabled(), mcap=f.memory_static_cap_bytes(),"
+            "mhead=f.memory_headroom_bytes(), scap=f.serve_memory_static_cap_bytes(),"
+            "shead=f.serve_memory_headroom_bytes())))")
     full_env = {k: v for k, v in os.environ.items() if not k.startswith("RETI_")}
     full_env.update(env)
     full_env["PYTHONPATH"] = ROOT
@@ -87,7 +90,8 @@ def test_flag_defaults_match_the_reference():
     d = _flags_in_subprocess({})
     assert d == dict(bf16_s=True, bf16_g=False, flash=True, twopass=True, minlen=2048, full=True,
                      res=False, serve=True, bt=256, blocks=128, per=128, pc=True, cap=4, chunk=0,
-                     split=128, simk=False, simv=False, par=128, pipe=True)
+                     split=128, simk=False, simv=False, par=128, pipe=True,
+                     guard=True, oom=True, mcap=None, mhead=2 << 30, scap=None, shead=2 << 30)
 
 
 def test_flag_overrides_and_precedence():
@@ -191,3 +195,18 @@ def test_resident_kv_bytes_and_layer_bytes():
             flags.layer_bytes(*bad, skv.DTYPE_BF16)
     with pytest.raises(skv.ConfigError):
         flags.layer_bytes(16, 16, 2, 256, 7)
+
+
+def test_memory_guard_flags_follow_the_reference():
+    # src/runtime_flags.rs:693-724, 773-792: the serve guard needs the shared guard; a cap of zero or
+    # an unparsable one is no cap; headrooms default to 2 GiB and accept surrounding blanks
+    d = _flags_in_subprocess({"RETI_MEMORY_GUARD": "0"})
+    assert (d["guard"], d["oom"]) == (False, False)
+    d = _flags_in_subprocess({"RETI_SERVE_OOM_GUARD": "off"})
+    assert (d["guard"], d["oom"]) == (True, False)
+    d = _flags_in_subprocess({"RETI_MEMORY_CAP_BYTES": " 1000000 ", "RETI_SERVE_MEMORY_CAP_BYTES": "0",
+                              "RETI_MEMORY_HEADROOM_BYTES": "0", "RETI_SERVE_MEMORY_HEADROOM_BYTES": "12x"})
+    assert (d["mcap"], d["scap"], d["mhead"], d["shead"]) == (1000000, None, 0, 2 << 30)
+    d = _flags_in_subprocess({"RETI_MEMORY_CAP_BYTES": "-5", "RETI_SERVE_MEMORY_CAP_BYTES": "68719476736",
+                              "RETI_SERVE_MEMORY_HEADROOM_BYTES": " 1073741824"})
+    assert (d["mcap"], d["scap"], d["shead"]) == (None, 1 << 36, 1 << 30)

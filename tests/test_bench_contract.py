@@ -57,6 +57,10 @@ def test_default_run_prints_one_json_line_with_the_agreed_keys():
     assert 0 <= d["checked_max_abs"] <= 1e-4
     # the restore leg carries the reference's state clone beside it
     assert d["restore"]["cpu_baseline"]["kind"] == "port" and d["restore"]["cpu_baseline"]["value"] > 0
+    # the reference's own SDPA length sweep
+    sweep = d["sdpa_sweep"]["rows"]
+    assert sorted({r["len"] for r in sweep}) == [1024, 4096, 16384, 32768] and {r["element"] for r in sweep} == {"f32", "bf16"}
+    assert all(r["us_per_call"] > 0 and r["gbps_effective"] > 0 and r["host_call_ms_per_call"] > 0 for r in sweep)
     # the further legs of the default run: configs[4] at batch 4 and the f32 element
     legs = d["legs"]
     for key, dtype in (("configs4_batch4", "bf16"), ("configs2_f32_element", "f32")):
