@@ -144,7 +144,6 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     // elements tid (and tid + THREADS where the head is wider than the workgroup) of the new
     // row of this kv head
     constexpr int NE = (P + THREADS - 1) / THREADS;
-    static_assert(!PRE || NE == 1, "the fused pre-KV step keeps one row element per thread");
     float k_rows[NE], v_rows[NE];
 #pragma unroll
     for (int u = 0; u < NE; ++u) {
@@ -155,11 +154,10 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             v_rows[u] = a.v_new[kvh * g.head_dim + tid + u * THREADS];
         }
     }
-    float &k_row = k_rows[0];
     // PRE: raw query rows of the group (and the raw k row, already in k_row)
     constexpr int PRE_U = PRE ? (16 * P + THREADS - 1) / THREADS : 1;
     float pre_q[PRE_U];
-    float pre_w0 = 1.0f, pre_w1 = 1.0f, pre_r = 0.0f;
+    float pre_w0[NE], pre_w1[NE], pre_r[NE];
     if (PRE) {
 #pragma unroll
         for (int u = 0; u < PRE_U; ++u) {
@@ -167,11 +165,13 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             const int r = e / P, c = e % P;
             pre_q[u] = (r < rows && c < g.head_dim) ? a.q[(long)(kvh * G + r) * q_stride + c] : 0.0f;
         }
-        if (tid < g.head_dim) {
-            if (a.q_norm_w) pre_w0 = a.q_norm_w[tid];
-            if (a.k_norm_w) pre_w1 = a.k_norm_w[tid];
+#pragma unroll
+        for (int u = 0; u < NE; ++u) {
+            const int d = tid + u * THREADS;
+            pre_w0[u] = (a.q_norm_w && d < g.head_dim) ? a.q_norm_w[d] : 1.0f;
+            pre_w1[u] = (a.k_norm_w && d < g.head_dim) ? a.k_norm_w[d] : 1.0f;
+            pre_r[u] = (a.rope && d < a.rope_dims) ? a.rope[d] : 0.0f;
         }
-        if (a.rope && tid < a.rope_dims) pre_r = a.rope[tid];
     }
 
     // Block-table entries of the next 64 iterations, one per lane.
@@ -238,12 +238,16 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
                 pre_sq[r * SQS + c] = sq_of(pre_q[u]);
             }
         }
-        if (tid < P) {
-            pre_raw[rows * PS + tid] = k_row;
-            pre_sq[rows * SQS + tid] = sq_of(k_row);
-            pre_wq[tid] = pre_w0;
-            pre_wk[tid] = pre_w1;
-            pre_rope[tid] = pre_r;
+#pragma unroll
+        for (int u = 0; u < NE; ++u) {
+            const int d = tid + u * THREADS;
+            if (d < P) {
+                pre_raw[rows * PS + d] = k_rows[u];
+                pre_sq[rows * SQS + d] = sq_of(k_rows[u]);
+                pre_wq[d] = pre_w0[u];
+                pre_wk[d] = pre_w1[u];
+                pre_rope[d] = pre_r[u];
+            }
         }
         __syncthreads();
         const int n_rows = rows + (appends ? 1 : 0);
@@ -264,7 +268,9 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             }
         }
         __syncthreads();
-        if (appends && tid < g.head_dim) k_row = pre_out[rows * PS + tid];
+#pragma unroll
+        for (int u = 0; u < NE; ++u)
+            if (appends && tid + u * THREADS < g.head_dim) k_rows[u] = pre_out[rows * PS + tid + u * THREADS];
     }
     if (appends) {
         // the page's physical id comes with the arguments: a table lookup here would wait for
@@ -697,11 +703,14 @@ static hipError_t launch_split(const DecodeArgs &a, hipStream_t s) {
 
 // head_dim 257..512 (global layers of Gemma-4-style models, src/config/accessors.rs:118-123):
 // the accumulators and one K and one V page alone are 256 registers, so the workgroup has
-// four wavefronts, one per SIMD with 512 registers each; no fused pre-KV variant.
+// four wavefronts, one per SIMD with 512 registers each (two row elements per thread in the
+// fused pre-KV step and the fused append).
 static hipError_t launch_split_wide(const DecodeArgs &a, hipStream_t s) {
-    if (a.pre) return hipErrorInvalidValue;
-    if (a.n_queries > 1 || a.g.gqa > 16) return launch_split_mq<512, 4, true, false>(a, s);
-    return launch_split_mq<512, 4, false, false>(a, s);
+    if (a.n_queries > 1 || a.g.gqa > 16) {
+        if (a.pre) return hipErrorInvalidValue;
+        return launch_split_mq<512, 4, true, false>(a, s);
+    }
+    return a.pre ? launch_split_mq<512, 4, false, true>(a, s) : launch_split_mq<512, 4, false, false>(a, s);
 }
 
 hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {

@@ -223,9 +223,9 @@ bool uses_flash(const skv_layer *L) { return skv_flag_flash_sdpa_enabled() && L-
 // on f32 layers where the f32 decode kernel serves the shape (head_dim up to 256, at most 16
 // heads per group).
 bool fused_append_built(const skv_layer *L) { return !L->g.f32 || (L->g.P <= 256 && L->g.gqa <= 16); }
-// The fused pre-KV step is built up to head_dim 256; wider heads take the separate
-// norm/rotation launches.
-bool wide_heads(const skv_layer *L) { return L->g.P > 256; }
+// The fused pre-KV step is built for bf16 layers up to head_dim 512 and for f32 layers up to
+// head_dim 256; wide f32 heads take the separate norm/rotation launches.
+bool wide_f32_heads(const skv_layer *L) { return L->g.f32 && L->g.P > 256; }
 
 // Arguments of the matrix-core attention kernel for the layer's current length.
 void fill_decode_args(const skv_layer *L, const float *q_dev, float *out_dev, size_t window_start,
@@ -1354,7 +1354,7 @@ static int32_t prekv_step(skv_layer *L, skv_stream stream, const skv_rope *rope,
                                            std::to_string(L->capacity) + " atteinte (overflow)");
     hipStream_t s = as_stream(stream);
     const bool fused = tuning().fused_append;
-    if (!fused || !uses_flash(L) || wide_heads(L) || L->g.gqa > 16) {
+    if (!fused || !uses_flash(L) || wide_f32_heads(L) || L->g.gqa > 16) {
         // the same step as separate launches: norm + rotation of q and k, append, attention, gate
         NormRopeArgs n{};
         n.x = q;

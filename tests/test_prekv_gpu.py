@@ -134,7 +134,9 @@ CASES = [
     ((4, 2, 16), 0, 3, 30, 4, 1.0e6, None, (True, True)),         # the reference's Gemma case: rope_dims = head_dim / 4
     ((8, 2, 64), 0, 0, 50, 64, 10000.0, 1.0, (False, False)),     # rotation only, from an empty cache
     ((6, 2, 96), 0, 20, 20, 32, 10000.0, None, (True, False)),    # q norm only, padded head_dim
-    ((8, 2, 512), 0, 300, 12, 128, 1.0e6, None, (True, True)),    # head_dim 512: norm/rotation as separate launches
+    ((8, 2, 512), 0, 300, 12, 128, 1.0e6, None, (True, True)),    # head_dim 512: two row elements per thread
+    ((16, 8, 512), 48, 10, 100, 512, 1.0e6, 300.0, (True, True)), # head_dim 512 on a ring layer, full rotation
+    ((8, 2, 384), 0, 4100, 8, 96, 1.0e6, None, (True, False)),    # head_dim 384 padded to 512, split-K
 ]
 
 
@@ -272,7 +274,8 @@ GATED = [
     ((16, 2, 256), 0, 3, 30, 64, 1.0e7),      # short cache: the split kernel applies the gate itself
     ((8, 4, 64), 32, 5, 80, 64, 10000.0),     # ring layer
     ((6, 2, 96), 0, 40, 10, 48, 10000.0),     # padded head_dim
-    ((4, 2, 512), 0, 100, 8, 128, 1.0e6),     # head_dim 512: every stage a launch of its own
+    ((4, 2, 512), 0, 100, 8, 128, 1.0e6),     # head_dim 512
+    ((16, 8, 512), 0, 2100, 6, 128, 1.0e6),   # head_dim 512, split-K with the gate in the merge
 ]
 
 
