@@ -58,3 +58,38 @@ def test_random_batch_matches_the_oracle(state, case):
         gk, gv = kv.read_rows_f32(m - keep, keep)
         assert np.array_equal(gk, cache.keys()[m - keep:]) and np.array_equal(gv, cache.values()[m - keep:])
         kv.close()
+
+
+def test_full_batch_of_sixteen_heads_per_group_at_head_dim_256(state):
+    """16 sequences (the most one launch takes) of q32/kv2/hd256 at about 600 rows: 320
+    four-wavefront workgroups, each with the largest exchange area the kernel has (16 query
+    heads x 256 columns per wavefront), more workgroups than the device holds at once."""
+    rng = np.random.default_rng(77)
+    q_heads, kv_heads, head_dim = 32, 2, 256
+    kv_dim, q_dim = kv_heads * head_dim, q_heads * head_dim
+    seqs = []
+    for i in range(16):
+        n = 590 + i
+        kv = state.full_attention_bf16(n + 8, q_heads, kv_heads, head_dim)
+        kv.set_block_table(rng.permutation(kv.pages()).astype(np.int32))
+        lay = oracle.layout(q_heads, kv_heads, head_dim)
+        cache = oracle.LayerKvCache("bf16r")
+        k0 = rng.standard_normal((n, kv_dim), dtype=np.float32)
+        v0 = rng.standard_normal((n, kv_dim), dtype=np.float32)
+        kv.seed(k0, v0, n)
+        cache.append_batch(k0, v0, lay)
+        seqs.append((kv, cache, lay))
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3):
+        rows = [(rng.standard_normal(kv_dim, dtype=np.float32), rng.standard_normal(kv_dim, dtype=np.float32),
+                 rng.standard_normal(q_dim, dtype=np.float32)) for _ in seqs]
+        dev = [[torch.from_numpy(a).cuda() for a in r] for r in rows]
+        outs = [torch.empty(q_dim, device="cuda") for _ in seqs]
+        skv.encode_decode_step_batch([s[0] for s in seqs], stream, [d[0].data_ptr() for d in dev],
+                                     [d[1].data_ptr() for d in dev], [d[2].data_ptr() for d in dev],
+                                     [o.data_ptr() for o in outs])
+        for (kv, cache, lay), (k, v, q), o in zip(seqs, rows, outs):
+            want = oracle.decode_step(cache, k, v, q, lay)
+            assert np.abs(o.cpu().numpy() - want).max() <= 1e-4
+    for kv, _, _ in seqs:
+        kv.close()
