@@ -468,8 +468,13 @@ def bench_config3(args, skv, torch, np, state, stream):
     # from an arena (DecodeResidentState::full_attention, src/decode_resident/attention.rs:26-108)
     # rather than allocating per request, and copies into memory that was never touched since
     # its allocation run at about half the rate.
-    max_tokens = len(shared) + 1024 + 512 + 16
+    n_decode = 128   # generated tokens per request (DEFAULT_MAX_TOKENS, src/bench_serve.rs:34)
+    max_tokens = len(shared) + 1024 + 512 + 16 + n_decode
     layers = make_layers(max_tokens, 1)
+    dq = torch.randn(nl, qh * hd, device=dev, dtype=torch.float32)
+    dk = torch.randn(nl, kv_dim, device=dev, dtype=torch.float32)
+    dv = torch.randn(nl, kv_dim, device=dev, dtype=torch.float32)
+    dout = torch.empty(nl, qh * hd, device=dev, dtype=torch.float32)
 
     def run_turn(tokens, seed):
         n = len(tokens)
@@ -528,6 +533,20 @@ def bench_config3(args, skv, torch, np, state, stream):
             if not (torch.equal(gk[:n], wk) and torch.equal(gv[:n], wv)):
                 raise RuntimeError("config 3: cache contents differ from the re-derived rows "
                                    "(layer %d, %d reused tokens)" % (i, reused))
+        # the request's decode phase on the KV side: n_decode tokens, each one fused append +
+        # attention step per layer over the prompt just restored and appended (decode_tok_s of
+        # bench-serve's RequestReport, src/bench_serve.rs:292-305, without the model around it)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n_decode):
+            for i, kv in enumerate(layers):
+                kv.encode_decode_step(stream, dk[i].data_ptr(), 0, dv[i].data_ptr(), 0, dq[i].data_ptr(),
+                                      dout[i].data_ptr())
+        e1.record()
+        torch.cuda.synchronize()
+        requests[-1]["generated_tokens"] = n_decode
+        requests[-1]["decode_kv_tok_s"] = round(n_decode / (e0.elapsed_time(e1) * 1e-3), 1)
         return reused
 
     requests = []
@@ -565,6 +584,7 @@ def bench_config3(args, skv, torch, np, state, stream):
                         "failed": sum(not r["ok"] for r in requests), "concurrency": 1,
                         "prefill_kv_p50_us": round(_percentile([r["prefill_kv_us"] for r in requests], 0.50), 1),
                         "prefill_kv_p95_us": round(_percentile([r["prefill_kv_us"] for r in requests], 0.95), 1),
+                        "decode_kv_tok_s_mean": round(sum(r["decode_kv_tok_s"] for r in requests) / len(requests), 1),
                         "prompt_tokens": tot["prompt"], "reused_prefix_tokens": tot["reused"],
                         "total_ms": round(wall * 1e3, 1)},
             "requests": requests},

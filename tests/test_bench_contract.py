@@ -112,3 +112,6 @@ def test_config3_report_counts_the_reused_tokens_the_reference_algorithm_reuses(
     assert rep["summary"]["reused_prefix_tokens"] == sum(w[1] for w in want) == d["reused_tokens"]
     assert rep["summary"]["prompt_tokens"] == sum(w[0] for w in want)
     assert all(q["restore_us"] > 0 for q in rep["requests"] if q["reused_prefix_tokens"])
+    # the decode phase of every request on the KV side (bench-serve's decode_tok_s, generated_tokens)
+    assert all(q["generated_tokens"] == 128 and q["decode_kv_tok_s"] > 0 for q in rep["requests"])
+    assert rep["summary"]["decode_kv_tok_s_mean"] > 0
