@@ -177,6 +177,10 @@ def test_snapshot_restore_and_hot_cache_on_f32_layers(state):
 
 
 def test_device_steps_on_f32_layers(state):
+    # wide f32 heads: norm and rotation, append and attention as launches of their own
+    run_prekv(state, (8, 2, 512), 0, 300, 20, 128, 1.0e6, None, (True, True), element="f32")
+    run_prekv(state, (4, 2, 384), 40, 10, 60, 96, 1.0e6, 300.0, (True, False), element="f32")
+    run_gated(state, (4, 2, 512), 0, 100, 20, 128, 1.0e6, element="f32")
     # the pre-KV and gated entry points are one launch pair on an f32 layer too (head_dim <= 256)
     run_prekv(state, (16, 2, 256), 0, 300, 6, 64, 1.0e7, None, (True, True), element="f32")
     run_prekv(state, (8, 2, 64), 40, 100, 30, 64, 1.0e6, None, (True, False), element="f32")
@@ -185,7 +189,12 @@ def test_device_steps_on_f32_layers(state):
 
 @pytest.mark.parametrize("dims,start,window", [((16, 2, 256), 0, 0), ((16, 2, 256), 4090, 0), ((32, 8, 128), 1000, 0),
                                                ((8, 2, 64), 15, 0), ((4, 1, 80), 31, 0), ((16, 8, 256), 100, 64),
-                                               ((16, 2, 256), 20000, 0)])
+                                               ((16, 2, 256), 20000, 0),
+                                               # shapes whose step is an append launch, then the kernel that also
+                                               # serves chunks: wide heads, padded wide heads, more than 16 heads per
+                                               # group, from empty, on a ring, split-K
+                                               ((16, 8, 512), 0, 0), ((4, 1, 320), 2040, 0), ((8, 2, 512), 9000, 0),
+                                               ((8, 2, 512), 40, 48), ((40, 2, 64), 500, 0), ((20, 1, 128), 3, 32)])
 def test_fused_decode_steps_on_f32_layers(state, dims, start, window):
     """skv_decode_step_device on an f32 layer is one launch pair: the attention kernel stores the
     new row itself and patches it into the registers of the wavefront that walks its page
