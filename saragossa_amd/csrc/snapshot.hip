@@ -17,7 +17,7 @@
 namespace skv {
 
 // ---- one launch copies up to COPY_MAX_PAGES pages of up to COPY_MAX_LAYERS layers --------
-constexpr int COPY_MAX_LAYERS = 56;
+constexpr int COPY_MAX_LAYERS = 48;
 constexpr int COPY_MAX_PAGES = 192;
 
 struct CopyLayer {
@@ -29,6 +29,7 @@ struct CopyLayer {
     uint32_t ring_pages;  // 0, or the ring's page count (logical page -> page % ring_pages)
     uint32_t first_page;  // logical pages below this one are skipped (rows a ring no longer holds)
     uint32_t pad;
+    uint64_t slot_stride; // bytes between this layer's pages of consecutive slots
 };
 
 struct CopyArgs {
@@ -36,7 +37,6 @@ struct CopyArgs {
     int32_t layer_page[COPY_MAX_PAGES]; // logical page inside every layer
     int32_t slot[COPY_MAX_PAGES];       // page slot inside the snapshot storage
     uint8_t *base;                      // snapshot storage
-    uint64_t slot_bytes;                // one 16-token page across all layers, K and V
     int n_layers;
     int n_pages;
     int to_snapshot; // 1: cache -> storage, 0: storage -> cache
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void page_copy_kernel(CopyArgs a) {
     const uint32_t tp = L.ring_pages ? lp % L.ring_pages : lp;
     const int page = L.table[tp];
     uint8_t *cache = reinterpret_cast<uint8_t *>(kv ? L.v_pool : L.k_pool) + (size_t)page * L.page_bytes;
-    uint8_t *store = a.base + (size_t)a.slot[pi] * a.slot_bytes + L.slot_off + (size_t)kv * L.page_bytes;
+    uint8_t *store = a.base + (size_t)a.slot[pi] * L.slot_stride + L.slot_off + (size_t)kv * L.page_bytes;
     const u32x4 *src = reinterpret_cast<const u32x4 *>(a.to_snapshot ? cache : store);
     u32x4 *dst = reinterpret_cast<u32x4 *>(a.to_snapshot ? store : cache);
     copy_stream(src, dst, (long)(L.page_bytes >> 4), threadIdx.x, 256);
@@ -158,23 +158,36 @@ struct SlotLayout {
     std::vector<uint32_t> page_bytes; // per layer
     std::vector<uint64_t> shape;      // per layer: what the bytes of a page mean
     std::vector<uint64_t> slot_off;
+    std::vector<uint64_t> slot_stride;
     uint64_t slot_bytes = 0;
+    bool layer_major = false;
 
     // kv heads, head_dim and element: two layers whose pages merely have the same size
     // (bf16 at head_dim 256 and f32 at 128, say) must not exchange pages
     static uint64_t shape_of(const skv_layer *L) {
         return ((uint64_t)L->g.kv_heads << 32) | ((uint64_t)L->g.head_dim << 1) | (uint64_t)(L->g.f32 & 1);
     }
-    void build(skv_layer *const *layers, size_t n) {
+    void build(skv_layer *const *layers, size_t n, size_t slots = 0, bool by_layer = false) {
         page_bytes.resize(n);
         shape.resize(n);
         slot_off.resize(n);
+        slot_stride.resize(n);
         slot_bytes = 0;
         for (size_t i = 0; i < n; ++i) {
             page_bytes[i] = (uint32_t)((size_t)layers[i]->g.page_elems * sizeof(uint16_t));
             shape[i] = shape_of(layers[i]);
             slot_off[i] = slot_bytes;
             slot_bytes += 2ull * page_bytes[i];
+        }
+        // Slot-major storage (a snapshot object): slot s holds one page of every layer, K then V,
+        // contiguously. Layer-major storage (the hot cache's pool): a layer's pages of all
+        // `slots` slots form one region, so the launches of a restore, which walk layer by
+        // layer, read from one region and write into one pool at a time (217-219 us against
+        // 228 us for 256 blocks of 36 layers; one-block snapshots cost the same either way).
+        layer_major = by_layer;
+        for (size_t i = 0; i < n; ++i) {
+            slot_stride[i] = by_layer ? 2ull * page_bytes[i] : slot_bytes;
+            if (by_layer) slot_off[i] *= slots;
         }
     }
     bool matches(skv_layer *const *layers, size_t n) const {
@@ -215,9 +228,8 @@ static int32_t copy_pages(const SlotLayout &lay, uint8_t *base, skv_layer *const
             a.n_layers = (int)nl;
             a.n_pages = (int)std::min<size_t>(COPY_MAX_PAGES, n_pages - p0);
             a.base = base;
-            a.slot_bytes = lay.slot_bytes;
             a.to_snapshot = to_snapshot ? 1 : 0;
-            a.layer_major = !to_snapshot && (size_t)a.n_pages >= layer_major_min_pages() ? 1 : 0;
+            a.layer_major = (!to_snapshot || lay.layer_major) && (size_t)a.n_pages >= layer_major_min_pages() ? 1 : 0;
             for (size_t i = 0; i < nl; ++i) {
                 skv_layer *L = layers[l0 + i];
                 CopyLayer &c = a.layers[i];
@@ -225,6 +237,7 @@ static int32_t copy_pages(const SlotLayout &lay, uint8_t *base, skv_layer *const
                 c.v_pool = L->v_pool;
                 c.table = L->table_dev;
                 c.slot_off = lay.slot_off[l0 + i];
+                c.slot_stride = lay.slot_stride[l0 + i];
                 c.page_bytes = lay.page_bytes[l0 + i];
                 c.ring_pages = L->g.ring_rows > 0 ? (uint32_t)L->n_pages : 0;
                 c.first_page = first_page ? first_page[l0 + i] : 0;
@@ -499,9 +512,9 @@ int32_t skv_hot_create(skv_ctx *ctx, size_t block_tokens, size_t capacity_blocks
     skv_hot *h = new skv_hot();
     h->ctx = ctx;
     h->index = new PrefixIndex(block_tokens, capacity_blocks, blocks_per_session);
-    h->layout.build(layers, n_layers);
     h->pages_per_block = block_tokens / 16;
     h->pool_slots = pool_blocks * h->pages_per_block;
+    h->layout.build(layers, n_layers, h->pool_slots, true);
     const size_t bytes = h->pool_slots * h->layout.slot_bytes;
     if (bytes) {
         hipError_t e = hipMalloc((void **)&h->pool, bytes);
