@@ -796,7 +796,7 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
     h->index->match_start(&walk, root);
     std::vector<int32_t> pages, slots;
     size_t done_blocks = 0; // blocks whose copies have been queued
-    size_t batch = any_ring ? (size_t)-1 : 20;
+    size_t batch = any_ring ? (size_t)-1 : 16;
     const size_t bt = h->index->block_tokens();
     // Once the first batch of copies is queued the layers' rows are being overwritten: an
     // error after that point leaves every layer empty (len 0) rather than with its old length
@@ -829,10 +829,10 @@ int32_t skv_hot_match_restore(skv_hot *h, skv_stream stream, const uint8_t root[
                             pages.size(), nullptr, false, as_stream(stream));
             done_blocks = chain.size();
             if (rc) return fail_emptied(rc);
-            // Hashing a block takes about 0.29 us, copying it (Qwen3-4B shape) about 0.76 us plus
-            // 6 us per launch: a batch 3.5 times the last is hashed while the last is copied, and
-            // a 4096-token prefix goes out in three launches (20, 70, 166 blocks).
-            batch = std::min<size_t>(batch * 7 / 2, COPY_MAX_PAGES);
+            // Hashing a block takes about 0.29 us, copying it (Qwen3-4B shape) about 0.72 us plus
+            // 6 us per launch: a batch four times the last is hashed while the last is copied, and
+            // a 4096-token prefix goes out in three launches (16, 64, 176 blocks).
+            batch = std::min<size_t>(batch * 4, COPY_MAX_PAGES);
         }
         if (!walk.alive) break;
     }
