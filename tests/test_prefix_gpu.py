@@ -176,6 +176,7 @@ class SimDecoder(pc.PromptDecoder):
     ((16, 2, 256), 2, 32, 128, 0.5, 1),  # two pages per hash block
     ((32, 8, 128), 3, 16, 256, 0.6, 8),  # several blocks prefilled and remembered per call
     ((32, 8, 128), 2, 16, 128, 0.15, 5), # a pool so small that blocks of one call evict each other
+    ((4, 1, 32), 52, 16, 128, 0.6, 4),   # more layers than one copy launch takes (48): two launches per batch
 ])
 def test_multi_turn_hot_cache_is_bit_exact_and_follows_reference_lru(state, dims, n_layers, bt,
                                                                      prefix, pool_frac,
