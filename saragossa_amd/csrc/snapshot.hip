@@ -179,10 +179,10 @@ struct SlotLayout {
             slot_off[i] = slot_bytes;
             slot_bytes += 2ull * page_bytes[i];
         }
-        // Slot-major storage (a snapshot object): slot s holds one page of every layer, K then V,
-        // contiguously. Layer-major storage (the hot cache's pool): a layer's pages of all
-        // `slots` slots form one region, so the launches of a restore, which walk layer by
-        // layer, read from one region and write into one pool at a time (217-219 us against
+        // Slot-major storage: slot s holds one page of every layer, K then V, contiguously.
+        // Layer-major storage (the hot cache's pool and the snapshot objects): a layer's pages
+        // of all `slots` slots form one region, so the launches of a restore, which walk layer
+        // by layer, read from one region and write into one pool at a time (217-219 us against
         // 228 us for 256 blocks of 36 layers; one-block snapshots cost the same either way).
         layer_major = by_layer;
         for (size_t i = 0; i < n; ++i) {
@@ -345,7 +345,7 @@ int32_t skv_snapshot_blocks(skv_ctx *ctx, skv_stream stream, skv_layer *const *l
     SKV_HIP(hipSetDevice(ctx->device));
     skv_snapshot *snap = new skv_snapshot();
     snap->ctx = ctx;
-    snap->layout.build(layers, n_layers);
+    snap->layout.build(layers, n_layers, n_blocks, true);
     snap->n_pages = n_blocks;
     snap->bytes = n_blocks * snap->layout.slot_bytes;
     if (snap->bytes) {
@@ -998,7 +998,7 @@ int32_t skv_prompt_cache_put(skv_prompt_cache *c, skv_stream stream, const uint6
         SKV_HIP(hipSetDevice(c->ctx->device));
         skv_snapshot *snap = new skv_snapshot();
         snap->ctx = c->ctx;
-        snap->layout.build(layers, n_layers);
+        snap->layout.build(layers, n_layers, n_blocks, true);
         snap->n_pages = n_blocks;
         snap->bytes = n_blocks * snap->layout.slot_bytes;
         if (snap->bytes) {
