@@ -133,6 +133,23 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     const int pb1 = page_lo + (int)(((unsigned)(split + 1) * span) / (unsigned)a.splits);
     // this wavefront walks pages pb0 + wave + it * WAVES, it = 0 .. n_it-1
     const int n_it = pb1 - pb0 > wave ? (pb1 - pb0 - wave + WAVES - 1) / WAVES : 0;
+    // Every other split, the last one among them, walks its pages starting from the middle of
+    // its range (rot .. n_it-1, then 0 .. rot-1); any order gives the same sums up to rounding.
+    // Two things are gained. The last split holds the newest page, the one the previous steps'
+    // appends wrote into, and is the split with a page more than the others when the pages do
+    // not divide: read at the end of that workgroup's chain, the newest page made it the
+    // slowest of the launch (176 against 167 us per token at 32768 rows of config 2, as much
+    // as the whole surplus page had been found to cost); read early, its latency is covered.
+    // And with pages laid out in order (an identity block table) all workgroups otherwise ask
+    // for addresses that share their middle bits at the same time (185 against 181 us). Only
+    // where every wavefront has two pages or more: on short launches (config 1: four or five
+    // pages per workgroup) it costs 2 %. The f32 kernel, tried the same way, lost 1.5 %.
+    const bool turns = ((split ^ (a.splits - 1)) & 1) == 0;
+    const int rot = (turns && pb1 - pb0 >= 2 * WAVES && n_it <= 64) ? (n_it >> 1) : 0;
+    auto turned = [&](int it) __attribute__((always_inline)) {
+        const int r = it + rot;
+        return r >= n_it ? r - n_it : r;
+    };
 
     // Fused append: the workgroup whose range holds the page of the new row rounds that
     // row to bf16, stores it into the pools for later steps and keeps it in LDS; the
@@ -181,6 +198,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         ids = it < n_it ? a.table[pb0 + wave + it * WAVES] : 0;
     };
     auto page_id = [&](int it) __attribute__((always_inline)) {
+        if (n_it <= 64) return __builtin_amdgcn_readlane(ids, turned(it)); // one register holds them all
         if ((it & 63) == 0 && it > 0) fetch_ids(it >> 6);
         return __builtin_amdgcn_readlane(ids, it & 63);
     };
@@ -219,7 +237,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     uint4 kr[KK], vr[KK];
     {
         typedef const __attribute__((address_space(4))) int32_t *const_i32_ptr;
-        const int pg = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(a.table))[min(pb0 + wave, max(page_hi - 1, 0))];
+        const int pg = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(a.table))[min(pb0 + wave + rot * WAVES, max(page_hi - 1, 0))];
         load_k<KK>(kr, a, pg, kvh, lane);
         load_v<KK>(vr, a, pg, kvh, lane);
     }
@@ -469,7 +487,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
     // Steady state is unconditional (the compiler can then wait for exactly the loads it
     // needs); the last page is peeled.
     for (int it = 0; it + 1 < n_it; ++it) {
-        const int pb = pb0 + wave + it * WAVES;
+        const int pb = pb0 + wave + turned(it) * WAVES;
         const int next = page_id(it + 1);
         patch_k(pb);
         const float4_t s = qk();
@@ -482,7 +500,7 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
         load_v<KK>(vr, a, next, kvh, lane);
     }
     if (n_it > 0) {
-        const int pb = pb0 + wave + (n_it - 1) * WAVES;
+        const int pb = pb0 + wave + turned(n_it - 1) * WAVES;
         patch_k(pb);
         const float4_t s = qk();
         short4_t ph, pl;
