@@ -135,7 +135,9 @@ hipError_t launch_iota(int32_t *dst, int n, hipStream_t s) {
 // an empty launch of the same shape.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(512) void probe_read_kernel(ProbeArgs a) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wavefront's number as a scalar: the block-table entries then come through the scalar
+    // unit and do not queue behind the other wavefronts' tile loads
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int split = blockIdx.x, kvh = blockIdx.y;
     const int pb0 = (int)(((long)split * a.n_pages) / a.splits);
     const int pb1 = (int)(((long)(split + 1) * a.n_pages) / a.splits);
@@ -149,11 +151,20 @@ __global__ __launch_bounds__(512) void probe_read_kernel(ProbeArgs a) {
         const u32x4_t *vp = reinterpret_cast<const u32x4_t *>(a.v_pool + tile);
         for (int u = lane; u < units; u += 64 * 8) {
             u32x4_t k[8], v[8];
+            if ((units & 511) == 0) {
+                // whole rounds of 512 units: constant offsets from one address per tile
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int at = min(u + i * 64, units - 1);
-                k[i] = __builtin_nontemporal_load(kp + at);
-                v[i] = __builtin_nontemporal_load(vp + at);
+                for (int i = 0; i < 8; ++i) {
+                    k[i] = __builtin_nontemporal_load(kp + u + i * 64);
+                    v[i] = __builtin_nontemporal_load(vp + u + i * 64);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int at = min(u + i * 64, units - 1);
+                    k[i] = __builtin_nontemporal_load(kp + at);
+                    v[i] = __builtin_nontemporal_load(vp + at);
+                }
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc ^= k[i].x ^ k[i].w ^ v[i].y ^ v[i].z;

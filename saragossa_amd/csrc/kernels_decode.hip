@@ -686,6 +686,137 @@ __global__ __launch_bounds__(256) void decode_merge_batch_kernel(DecodeBatchArgs
     decode_merge_body<MERGE_PER_LANE>(a);
 }
 
+// ------------------------------------------------------------------------------------
+// The same merge with one wavefront per (query head, 16 columns) and nothing shared between
+// wavefronts: the 64 lanes are 4 column lanes (four columns each, one 16-byte load per
+// split) x 16 split lanes. Every lane asks for o, m and l of its splits at once; the
+// maximum and the sums go across the split lanes with row rotations and row swaps in the
+// vector unit, so that no lane waits at a barrier or for LDS. Row offsets are 32-bit: the
+// launcher checks that one kv head's partials stay below 4 GiB and that head_dim is a
+// multiple of four.
+// ------------------------------------------------------------------------------------
+struct MergeArgs {
+    const float *part_o;
+    const float *part_m;
+    const float *part_l;
+    float *out;
+    const float *gate;
+    int splits_total, n_queries, gqa, q_heads, head_dim, q_head_stride;
+    int waves; // wavefronts (column groups) per workgroup
+};
+
+template <int CTRL>
+__device__ __forceinline__ float row_rotated(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// over the 16 split lanes (lane bits 2..5) of one column lane, every lane receiving the result
+__device__ __forceinline__ float split_lanes_max(float v) {
+    v = fmaxf(v, row_rotated<0x124>(v)); // row_ror:4
+    v = fmaxf(v, row_rotated<0x128>(v)); // row_ror:8
+    return rows_max(v);
+}
+__device__ __forceinline__ float split_lanes_sum(float v) {
+    v += row_rotated<0x124>(v);
+    v += row_rotated<0x128>(v);
+    return rows_sum(v);
+}
+
+template <int PER>
+__device__ __forceinline__ void merge_wave_body(const MergeArgs &a, int kvh, int slot, int cg) {
+    const int lane = threadIdx.x & 63;
+    const int c4 = lane & 3, g = lane >> 2;
+    const int n_slots = a.n_queries * a.gqa;
+    const int col = cg * 16 + c4 * 4;
+    const bool col_ok = col < a.head_dim;
+    const long base = ((long)kvh * a.splits_total) * n_slots + slot;
+    const char *pm = reinterpret_cast<const char *>(a.part_m + base);
+    const char *pl = reinterpret_cast<const char *>(a.part_l + base);
+    const char *po = reinterpret_cast<const char *>(a.part_o + base * a.head_dim);
+    const uint32_t ml_stride = (uint32_t)n_slots * 4u;
+    const uint32_t o_stride = ml_stride * (uint32_t)a.head_dim;
+    const uint32_t g0 = g < a.splits_total ? (uint32_t)g : 0u;
+    const uint32_t ml0 = g0 * ml_stride;
+    const uint32_t o0 = g0 * o_stride + (col_ok ? (uint32_t)col * 4u : 0u);
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    f32x4_t ov[PER];
+    float mv[PER], lv[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const bool ok = g + 16 * i < a.splits_total;
+        const uint32_t mo = ok ? ml0 + (uint32_t)(16 * i) * ml_stride : ml0;
+        const uint32_t oo = ok ? o0 + (uint32_t)(16 * i) * o_stride : o0;
+        mv[i] = *reinterpret_cast<const float *>(pm + mo);
+        lv[i] = *reinterpret_cast<const float *>(pl + mo);
+        ov[i] = *reinterpret_cast<const f32x4_t *>(po + oo);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        if (g + 16 * i >= a.splits_total) mv[i] = -INFINITY;
+        mx = fmaxf(mx, mv[i]);
+    }
+    mx = split_lanes_max(mx);
+    const float m_safe = mx == -INFINITY ? 0.0f : mx;
+    f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    float lsum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const float w = fast_exp2(mv[i] - m_safe); // 0 for the splits beyond the last
+        acc += w * ov[i];
+        lsum += w * lv[i];
+    }
+    acc.x = split_lanes_sum(acc.x);
+    acc.y = split_lanes_sum(acc.y);
+    acc.z = split_lanes_sum(acc.z);
+    acc.w = split_lanes_sum(acc.w);
+    lsum = split_lanes_sum(lsum);
+    if (g == 0 && col_ok) {
+        const int qi = a.n_queries == 1 ? 0 : slot / a.gqa;
+        const long h = (long)qi * a.q_heads + kvh * a.gqa + (slot - qi * a.gqa); // output row
+        f32x4_t r = {acc.x / lsum, acc.y / lsum, acc.z / lsum, acc.w / lsum};
+        if (a.gate && a.n_queries == 1) {
+            const float *gp = a.gate + h * (a.q_head_stride > 0 ? a.q_head_stride : a.head_dim) + col;
+            r.x *= sigmoid_gate(gp[0]);
+            r.y *= sigmoid_gate(gp[1]);
+            r.z *= sigmoid_gate(gp[2]);
+            r.w *= sigmoid_gate(gp[3]);
+        }
+        *reinterpret_cast<f32x4_t *>(a.out + h * a.head_dim + col) = r;
+    }
+}
+
+// grid (column groups / wavefronts per workgroup, query slots, kv heads)
+template <int PER>
+__global__ __launch_bounds__(256) void decode_merge_wave_kernel(MergeArgs a) {
+    // a wavefront beyond the last column group goes through the motions on column 0 and
+    // stores nothing: no early exit, so that every kernel argument is asked for at once
+    const int cg = (int)blockIdx.x * a.waves + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    merge_wave_body<PER>(a, blockIdx.z, blockIdx.y, cg);
+}
+
+// Several sequences of one geometry, one query row each: grid (column groups, query heads,
+// sequences); a sequence with a single split already has its context.
+template <int PER>
+__global__ __launch_bounds__(64) void decode_merge_wave_batch_kernel(DecodeBatchArgs b) {
+    const DecodeArgs &d = b.seq[blockIdx.z];
+    if (d.splits_total <= 1) return;
+    MergeArgs a;
+    a.part_o = d.part_o;
+    a.part_m = d.part_m;
+    a.part_l = d.part_l;
+    a.out = d.out;
+    a.gate = d.gate;
+    a.splits_total = d.splits_total;
+    a.n_queries = 1;
+    a.gqa = d.g.gqa;
+    a.q_heads = d.g.q_heads;
+    a.head_dim = d.g.head_dim;
+    a.q_head_stride = d.q_head_stride;
+    a.waves = 1;
+    const int kvh = (int)blockIdx.y / d.g.gqa;
+    merge_wave_body<PER>(a, kvh, (int)blockIdx.y - kvh * d.g.gqa, blockIdx.x);
+}
+
 template <int P, int WAVES, bool MQ, bool PRE>
 static hipError_t launch_split_mq(const DecodeArgs &a, hipStream_t s) {
     constexpr int KK = P / 32;
@@ -746,7 +877,46 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t s) {
     return launch_merge(a, s);
 }
 
+// Whether the wavefront merge serves these partials: 16-byte column loads, 32-bit offsets
+// within a kv head, and a grid that fits.
+static bool merge_wave_fits(const DecodeArgs &a) {
+    const uint64_t n_slots = (uint64_t)a.n_queries * a.g.gqa;
+    return a.g.head_dim % 4 == 0 && (uint64_t)a.splits_total * n_slots * a.g.head_dim * 4 < (1ull << 32) &&
+           n_slots <= 65535 && a.g.kv_heads <= 65535 && a.splits_total <= 16 * MERGE_PER_LANE_MAX &&
+           ((uintptr_t)a.part_o & 15) == 0 && ((uintptr_t)a.out & 15) == 0;
+}
+
+static hipError_t launch_merge_wave(const DecodeArgs &a, hipStream_t s) {
+    MergeArgs m;
+    m.part_o = a.part_o;
+    m.part_m = a.part_m;
+    m.part_l = a.part_l;
+    m.out = a.out;
+    m.gate = a.gate;
+    m.splits_total = a.splits_total;
+    m.n_queries = a.n_queries;
+    m.gqa = a.g.gqa;
+    m.q_heads = a.g.q_heads;
+    m.head_dim = a.g.head_dim;
+    m.q_head_stride = a.q_head_stride;
+    const int n_slots = a.n_queries * a.g.gqa;
+    const int n_cg = (a.g.head_dim + 15) / 16;
+    // one wavefront per workgroup while that still leaves few workgroups, else four
+    const int waves = (long)n_cg * n_slots * a.g.kv_heads <= 1024 ? 1 : 4;
+    m.waves = waves;
+    dim3 grid((unsigned)((n_cg + waves - 1) / waves), (unsigned)n_slots, (unsigned)a.g.kv_heads);
+    const dim3 block((unsigned)(64 * waves));
+    const int per = (a.splits_total + 15) / 16;
+    if (per <= 1) hipLaunchKernelGGL(decode_merge_wave_kernel<1>, grid, block, 0, s, m);
+    else if (per <= 2) hipLaunchKernelGGL(decode_merge_wave_kernel<2>, grid, block, 0, s, m);
+    else if (per <= 4) hipLaunchKernelGGL(decode_merge_wave_kernel<4>, grid, block, 0, s, m);
+    else if (per <= 8) hipLaunchKernelGGL(decode_merge_wave_kernel<8>, grid, block, 0, s, m);
+    else hipLaunchKernelGGL(decode_merge_wave_kernel<16>, grid, block, 0, s, m);
+    return hipGetLastError();
+}
+
 hipError_t launch_merge(const DecodeArgs &a, hipStream_t s) {
+    if (merge_wave_fits(a)) return launch_merge_wave(a, s);
     dim3 mgrid((unsigned)(a.g.kv_heads * a.n_queries * a.g.gqa), (unsigned)((a.g.head_dim + 15) / 16));
     const int per_lane = (a.splits_total + 15) / 16;
     if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_kernel<1>, mgrid, dim3(256), 0, s, a);
@@ -799,8 +969,19 @@ hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t 
     default: break;
     }
     if (e != hipSuccess || max_splits == 1) return e;
-    dim3 mgrid((unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)((a0.g.head_dim + 15) / 16), (unsigned)n_seq);
     const int per_lane = (max_splits + 15) / 16;
+    bool wave_merge = a0.g.kv_heads * a0.g.gqa <= 65535;
+    for (int i = 0; i < n_seq; ++i) wave_merge = wave_merge && b.seq[i].n_queries == 1 && merge_wave_fits(b.seq[i]);
+    if (wave_merge) {
+        dim3 grid((unsigned)((a0.g.head_dim + 15) / 16), (unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)n_seq);
+        if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<1>, grid, dim3(64), 0, s, b);
+        else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<2>, grid, dim3(64), 0, s, b);
+        else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<4>, grid, dim3(64), 0, s, b);
+        else if (per_lane <= 8) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<8>, grid, dim3(64), 0, s, b);
+        else hipLaunchKernelGGL(decode_merge_wave_batch_kernel<16>, grid, dim3(64), 0, s, b);
+        return hipGetLastError();
+    }
+    dim3 mgrid((unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)((a0.g.head_dim + 15) / 16), (unsigned)n_seq);
     if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_batch_kernel<1>, mgrid, dim3(256), 0, s, b);
     else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_batch_kernel<2>, mgrid, dim3(256), 0, s, b);
     else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_batch_kernel<4>, mgrid, dim3(256), 0, s, b);
