@@ -709,6 +709,16 @@ template <int CTRL>
 __device__ __forceinline__ float row_rotated(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
+// the value that lane K of each group of four lanes holds
+__device__ __forceinline__ float quad_lane(float v, int k) {
+    const int x = __float_as_int(v);
+    switch (k) { // k is a constant wherever this is used: one instruction
+    case 0: return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x00, 0xf, 0xf, false));
+    case 1: return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0x55, 0xf, 0xf, false));
+    case 2: return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0xaa, 0xf, 0xf, false));
+    default: return __int_as_float(__builtin_amdgcn_update_dpp(0, x, 0xff, 0xf, 0xf, false));
+    }
+}
 // over the 16 split lanes (lane bits 2..5) of one column lane, every lane receiving the result
 __device__ __forceinline__ float split_lanes_max(float v) {
     v = fmaxf(v, row_rotated<0x124>(v)); // row_ror:4
@@ -739,20 +749,34 @@ __device__ __forceinline__ void merge_wave_body(const MergeArgs &a, int kvh, int
     const uint32_t o0 = g0 * o_stride + (col_ok ? (uint32_t)col * 4u : 0u);
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
     f32x4_t ov[PER];
-    float mv[PER], lv[PER];
+    // m and l of a split are the same for the four column lanes: each of them asks for a
+    // quarter of the splits' pairs and hands them to the other three below
+    constexpr int NML = (PER + 3) / 4;
+    float mq[NML], lq[NML];
+#pragma unroll
+    for (int j = 0; j < NML; ++j) {
+        const int i = c4 + 4 * j;
+        const bool ok = i < PER && g + 16 * i < a.splits_total;
+        const uint32_t mo = ok ? ml0 + (uint32_t)(16 * i) * ml_stride : ml0;
+        mq[j] = *reinterpret_cast<const float *>(pm + mo);
+        lq[j] = *reinterpret_cast<const float *>(pl + mo);
+        if (!ok) {
+            mq[j] = -INFINITY;
+            lq[j] = 0.0f;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const bool ok = g + 16 * i < a.splits_total;
-        const uint32_t mo = ok ? ml0 + (uint32_t)(16 * i) * ml_stride : ml0;
         const uint32_t oo = ok ? o0 + (uint32_t)(16 * i) * o_stride : o0;
-        mv[i] = *reinterpret_cast<const float *>(pm + mo);
-        lv[i] = *reinterpret_cast<const float *>(pl + mo);
         ov[i] = *reinterpret_cast<const f32x4_t *>(po + oo);
     }
+    float mv[PER], lv[PER];
     float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        if (g + 16 * i >= a.splits_total) mv[i] = -INFINITY;
+        mv[i] = quad_lane(mq[i >> 2], i & 3);
+        lv[i] = quad_lane(lq[i >> 2], i & 3);
         mx = fmaxf(mx, mv[i]);
     }
     mx = split_lanes_max(mx);
