@@ -818,10 +818,10 @@ __global__ __launch_bounds__(256) void decode_merge_wave_kernel(MergeArgs a) {
     merge_wave_body<PER>(a, blockIdx.z, blockIdx.y, cg);
 }
 
-// Several sequences of one geometry, one query row each: grid (column groups, query heads,
-// sequences); a sequence with a single split already has its context.
+// Several sequences of one geometry, one query row each: grid (pairs of column groups, query
+// heads, sequences); a sequence with a single split already has its context.
 template <int PER>
-__global__ __launch_bounds__(64) void decode_merge_wave_batch_kernel(DecodeBatchArgs b) {
+__global__ __launch_bounds__(128) void decode_merge_wave_batch_kernel(DecodeBatchArgs b) {
     const DecodeArgs &d = b.seq[blockIdx.z];
     if (d.splits_total <= 1) return;
     MergeArgs a;
@@ -836,9 +836,10 @@ __global__ __launch_bounds__(64) void decode_merge_wave_batch_kernel(DecodeBatch
     a.q_heads = d.g.q_heads;
     a.head_dim = d.g.head_dim;
     a.q_head_stride = d.q_head_stride;
-    a.waves = 1;
+    a.waves = 2;
     const int kvh = (int)blockIdx.y / d.g.gqa;
-    merge_wave_body<PER>(a, kvh, (int)blockIdx.y - kvh * d.g.gqa, blockIdx.x);
+    const int cg = (int)blockIdx.x * 2 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    merge_wave_body<PER>(a, kvh, (int)blockIdx.y - kvh * d.g.gqa, cg);
 }
 
 template <int P, int WAVES, bool MQ, bool PRE>
@@ -925,8 +926,11 @@ static hipError_t launch_merge_wave(const DecodeArgs &a, hipStream_t s) {
     m.q_head_stride = a.q_head_stride;
     const int n_slots = a.n_queries * a.g.gqa;
     const int n_cg = (a.g.head_dim + 15) / 16;
-    // one wavefront per workgroup while that still leaves few workgroups, else four
-    const int waves = (long)n_cg * n_slots * a.g.kv_heads <= 1024 ? 1 : 4;
+    // Two wavefronts per workgroup, i.e. two neighbouring column groups on one compute unit,
+    // so that the 128-byte lines of the partials are fetched once and not once per half
+    // (FETCH_SIZE of the merge: 2235 KiB against 4277 KiB with one wavefront per workgroup, same
+    // time); four where the grid is large anyway (four on the decode step: 0.3 us slower).
+    const int waves = (long)n_cg * n_slots * a.g.kv_heads <= 1024 ? 2 : 4;
     m.waves = waves;
     dim3 grid((unsigned)((n_cg + waves - 1) / waves), (unsigned)n_slots, (unsigned)a.g.kv_heads);
     const dim3 block((unsigned)(64 * waves));
@@ -997,12 +1001,12 @@ hipError_t launch_decode_batch(const DecodeBatchArgs &b, int n_seq, hipStream_t 
     bool wave_merge = a0.g.kv_heads * a0.g.gqa <= 65535;
     for (int i = 0; i < n_seq; ++i) wave_merge = wave_merge && b.seq[i].n_queries == 1 && merge_wave_fits(b.seq[i]);
     if (wave_merge) {
-        dim3 grid((unsigned)((a0.g.head_dim + 15) / 16), (unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)n_seq);
-        if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<1>, grid, dim3(64), 0, s, b);
-        else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<2>, grid, dim3(64), 0, s, b);
-        else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<4>, grid, dim3(64), 0, s, b);
-        else if (per_lane <= 8) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<8>, grid, dim3(64), 0, s, b);
-        else hipLaunchKernelGGL(decode_merge_wave_batch_kernel<16>, grid, dim3(64), 0, s, b);
+        dim3 grid((unsigned)(((a0.g.head_dim + 15) / 16 + 1) / 2), (unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)n_seq);
+        if (per_lane <= 1) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<1>, grid, dim3(128), 0, s, b);
+        else if (per_lane <= 2) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<2>, grid, dim3(128), 0, s, b);
+        else if (per_lane <= 4) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<4>, grid, dim3(128), 0, s, b);
+        else if (per_lane <= 8) hipLaunchKernelGGL(decode_merge_wave_batch_kernel<8>, grid, dim3(128), 0, s, b);
+        else hipLaunchKernelGGL(decode_merge_wave_batch_kernel<16>, grid, dim3(128), 0, s, b);
         return hipGetLastError();
     }
     dim3 mgrid((unsigned)(a0.g.kv_heads * a0.g.gqa), (unsigned)((a0.g.head_dim + 15) / 16), (unsigned)n_seq);
