@@ -48,7 +48,7 @@ WORKLOADS = {
 # by what the counters read for a copy of known size (the method and the raw readings are in
 # profiles/decode_split_kernel_config2.md). Not measurable from inside this process, so it is
 # a recorded figure, present only for the workload it was taken on.
-MEASURED_TRAFFIC_BYTES = {2: 70185 * 1024}
+MEASURED_TRAFFIC_BYTES = {2: 70160 * 1024}
 
 
 # What the matrix pipes sustain for the prefill kernel's product stream when nothing else is in
@@ -1008,11 +1008,11 @@ def decode_bench(args, skv, torch, np, state, main_leg):
         "checked_max_abs": checked_max_abs,
         "checked": "context of layer 0 after the last timed step vs float64 softmax attention (torch) over "
                    "the rows read back from its cache; the run fails above 1e-4",
-        "roofline": {"bound": "hbm", "kernel": ("f32_split_kernel<%d> + decode_merge_kernel (one attention launch per "
+        "roofline": {"bound": "hbm", "kernel": ("f32_split_kernel<%d> + decode_merge_wave_kernel (one attention launch per "
                                                 "sequence, average over the layers)" if args.element == "f32" else
-                                                "decode_split_kernel<%d,8> + decode_merge_kernel (one attention launch, "
+                                                "decode_split_kernel<%d,8> + decode_merge_wave_kernel (one attention launch, "
                                                 "average over the layers)" if B == 1 else
-                                                "decode_split_batch_kernel<%d,8> + decode_merge_batch_kernel (one launch pair "
+                                                "decode_split_batch_kernel<%d,8> + decode_merge_wave_batch_kernel (one launch pair "
                                                 "per layer covers the batch, average over the layers)")
                                                % (128 if hd <= 128 else 256),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
