@@ -70,6 +70,19 @@ def test_attention_decode_other_shapes(state, dims, n):
     run_attention_case(state, n, *dims)
 
 
+@pytest.mark.parametrize("dims", [
+    (4, 2, 18), (6, 1, 30),   # head_dim not a multiple of four: the merge that reduces through LDS
+    (6, 2, 72),               # five column groups: the last merge workgroup has an idle wavefront
+    (3, 1, 8), (2, 2, 4),     # fewer columns than a column group
+    (16, 16, 64),             # one head per group
+])
+@pytest.mark.parametrize("n", [40, 700, 5000])
+def test_attention_decode_merge_paths(state, dims, n):
+    """Split counts from two to the device's fill (n = 40: two or three pages) over the head
+    widths that take the merge kernel's less common paths."""
+    run_attention_case(state, n, *dims)
+
+
 def test_qwen_uniform_attention_decode_is_byte_exact_single_key(state):
     # src/decode_resident/tests.rs:1356-1385: one key -> softmax is exactly 1, context == V row
     q_heads, kv_heads, head_dim = 4, 2, 16
