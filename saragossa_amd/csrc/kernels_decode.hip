@@ -404,8 +404,12 @@ __device__ __forceinline__ void decode_split_body(const DecodeArgs &a, const int
             pl[i] = (short)lb;
         }
         l_run = l_run * alpha + psum;
+        // A slot that has seen no key yet holds zeros: no rescale for it (the first page of
+        // every wavefront would otherwise walk all its accumulator registers for nothing, which
+        // on a launch of one page per wavefront is a visible part of the whole).
+        const bool rescale = alpha != 1.0f && m_run != -INFINITY;
         m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+        if (__builtin_amdgcn_ballot_w64(rescale)) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) o[t] *= alpha;
         }

@@ -260,8 +260,9 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
             psum += pv[e];
         }
         l_run = l_run * alpha + psum;
+        const bool rescale = alpha != 1.0f && m_run != -INFINITY; // a slot without a key so far holds zeros
         m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+        if (__builtin_amdgcn_ballot_w64(rescale)) {
 #pragma unroll
             for (int c = 0; c < NT; ++c) o[c] *= alpha;
         }
@@ -349,8 +350,9 @@ __global__ __launch_bounds__(256) void f32_split_kernel(DecodeArgs a) {
                     psum += pv[e];
                 }
                 l_run = l_run * alpha + psum;
+                const bool rescale = alpha != 1.0f && m_run != -INFINITY; // a slot without a key so far holds zeros
                 m_run = m_new;
-                if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+                if (__builtin_amdgcn_ballot_w64(rescale)) {
 #pragma unroll
                     for (int c = 0; c < NT; ++c) o[c] *= alpha;
                 }
@@ -692,8 +694,9 @@ __device__ __forceinline__ void f32_decode_body(const DecodeArgs &a, const int s
             psum += pv[e];
         }
         l_run = l_run * alpha + psum;
+        const bool rescale = alpha != 1.0f && m_run != -INFINITY; // a slot without a key so far holds zeros
         m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {
+        if (__builtin_amdgcn_ballot_w64(rescale)) {
 #pragma unroll
             for (int c = 0; c < NT; ++c) o[c] *= alpha;
         }
