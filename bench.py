@@ -275,24 +275,46 @@ def bench_prefill(skv, torch, np, state, stream, element="bf16"):
         k = torch.randn(chunk, kv_dim, device=dev, generator=gen)
         v = torch.randn(chunk, kv_dim, device=dev, generator=gen)
         o = torch.empty(chunk, q_dim, device=dev)
-        ts = []
-        for it in range(13):
-            kv.truncate(base)
+        def call():
+            kv.truncate(base)  # host bookkeeping only
+            kv.encode_prefill_rows(stream, q.data_ptr(), k.data_ptr(), v.data_ptr(), chunk, o.data_ptr())
+
+        def timed(calls):
             e0 = torch.cuda.Event(enable_timing=True)
             e1 = torch.cuda.Event(enable_timing=True)
             e0.record()
-            kv.encode_prefill_rows(stream, q.data_ptr(), k.data_ptr(), v.data_ptr(), chunk, o.data_ptr())
+            for _ in range(calls):
+                call()
             e1.record()
+            return e0, e1
+
+        # (a) one call at a time on a GPU that has just been idle, the way the kernel traces
+        # under profiles/ see it
+        single = []
+        for it in range(8):
+            torch.cuda.synchronize()
+            e0, e1 = timed(1)
             torch.cuda.synchronize()
             if it >= 3:
-                ts.append(e0.elapsed_time(e1) * 1e3)
-        ts.sort()
+                single.append(e0.elapsed_time(e1) * 1e3)
+        single.sort()
+        # (b) a stream of calls, like the chunks of a long prompt: this matrix-core-bound kernel
+        # keeps getting faster for some 40 ms of uninterrupted work (the device's clock
+        # management; the HBM-bound decode launches show no such drift), so about 70 ms of calls
+        # run untimed first, then 12 groups of four calls back to back
+        warm = max(16, min(int(70e3 / max(single[len(single) // 2], 1.0)), 2000))
+        for _ in range(warm):
+            call()
+        groups = [timed(4) for _ in range(12)]
+        torch.cuda.synchronize()
+        ts = sorted(e0.elapsed_time(e1) * 1e3 / 4 for e0, e1 in groups)
         us = ts[len(ts) // 2]
         keys = sum(base + i + 1 for i in range(chunk))
         flops = 4 * keys * q_dim
-        row = {"workload": "%s, %s element: %d-row chunk over %d cached rows (append + attention + merge)"
+        row = {"workload": "%s, %s element: %d-row chunk over %d cached rows (append + attention + merge; a stream of calls, four per event pair, after 70 ms of them)"
                            % (name, element, chunk, base),
-               "us": round(us, 1), "algorithmic_tflops": round(flops / us / 1e6, 1)}
+               "us": round(us, 1), "us_single_call_from_idle": round(single[len(single) // 2], 1),
+               "algorithmic_tflops": round(flops / us / 1e6, 1)}
         if f32:
             row["frac_of_f32_mfma_peak"] = round(flops / us / 1e6 / 157.3, 4)
         else:
