@@ -449,9 +449,14 @@ __global__ __launch_bounds__(256) void merge_rows_kernel(DecodeArgs a) {
     const int kvh = (int)(ks / n_slots);
     const int slot = (int)(ks - (long)kvh * n_slots);
     const long base = ((long)kvh * a.splits_total) * n_slots + slot;
+    // Up to four splits (the usual case: a chunk's tiles fill the device with few splits) are
+    // one round trip: the maximum comes from the m values that the round below loads anyway.
+    // More splits take a pass over m first.
+    const bool one_round = a.splits_total <= 4;
     float mx = -INFINITY;
-    for (int sp = 0; sp < a.splits_total; ++sp) mx = fmaxf(mx, a.part_m[base + (long)sp * n_slots]);
-    const float m_safe = mx == -INFINITY ? 0.0f : mx;
+    if (!one_round)
+        for (int sp = 0; sp < a.splits_total; ++sp) mx = fmaxf(mx, a.part_m[base + (long)sp * n_slots]);
+    float m_safe = mx == -INFINITY ? 0.0f : mx;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float lsum = 0.0f;
     const bool vec_ok = (g.head_dim & 3) == 0;
@@ -473,6 +478,10 @@ __global__ __launch_bounds__(256) void merge_rows_kernel(DecodeArgs a) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) v[u][i] = c4 + i < g.head_dim ? po[i] : 0.0f;
             }
+        }
+        if (one_round) {
+            mx = fmaxf(fmaxf(w[0], w[1]), fmaxf(w[2], w[3])); // repeats of the last split do not move it
+            m_safe = mx == -INFINITY ? 0.0f : mx;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
