@@ -53,10 +53,11 @@ MEASURED_TRAFFIC_BYTES = {2: 70160 * 1024}
 
 # What the matrix pipes sustain for the prefill kernel's product stream when nothing else is in
 # the kernel: 16x16x32 bf16 products with every operand in registers, on random operand values
-# (the clock under the matrix pipes drops when operand bits toggle), measured once with a
-# stand-alone product-stream program on one MI355X. A recorded figure, like the traffic above;
-# the published peak stays the roofline's `peak`.
-MFMA_STREAM_RANDOM_TFLOPS = 1580.0
+# (the clock under the matrix pipes drops when operand bits toggle), measured with a
+# stand-alone product-stream program on one MI355X in a stream of launches, like the prefill
+# leg's `us` (1732 with the launches one at a time; 1580 on the box of an earlier recording).
+# A recorded figure, like the traffic above; the published peak stays the roofline's `peak`.
+MFMA_STREAM_RANDOM_TFLOPS = 1783.0
 
 def algorithmic_bytes(rows: int, kv_dim: int, q_dim: int, with_append: bool, elem_bytes: int = 2) -> int:
     """Bytes one layer's decode step has to move: K and V once (in the cache's element: 2 bytes
