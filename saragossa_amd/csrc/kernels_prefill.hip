@@ -236,6 +236,7 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
 
     // ---- page copies: memory -> registers -> LDS -------------------------------------
     const int n_steps = (n_it + PG - 1) / PG;
+    constexpr int FETCH_PAIR = PG / 2 - 1; // in front of the step's last pair
     uint4 stage[PG][LOAD_U];
     // (a split without pages still reads one valid page, and writes empty partials below)
     fetch_step<P, PG, THREADS>(stage, a, pb0, 0, n_it, kvh, tid);
@@ -243,14 +244,20 @@ __global__ __launch_bounds__(WAVES * 64) void prefill_tile_kernel(DecodeArgs a) 
     __syncthreads();
 
     for (int step = 0; step < n_steps; ++step) {
-      // unconditional: after the last step this re-reads its pages into the idle buffer
-      fetch_step<P, PG, THREADS>(stage, a, pb0, min(step + 1, n_steps - 1), n_it, kvh, tid);
+      // The next step's pages are asked for in front of the last pair of this step, not at its
+      // top: the copies still land before store_step needs them, and the staging registers are
+      // live for less of the step (a stream of calls, same box each: config 2 shape 450 against
+      // 466 us and 470.6 against 480.3; config 1 shape, four pairs per step, 56.8 in front of the
+      // last pair, 57.4 and 57.9 in front of the third and second, 57.75 at the top; inside the
+      // last pair, after its scores or its softmax, 481-483 against 475 at config 2 shape).
+      // Unconditional: after the last step this re-reads its pages into the idle buffer.
       // Pages are consumed in pairs (A, B): the PV product then contracts over 32 keys with
       // the k index of lane group j, element e meaning key 4j+e of page A (e < 4) or key
       // 4j+e-4 of page B, which is exactly how the two S^T tiles and the two V tiles already
       // sit in the lanes.
 #pragma unroll
       for (int pp = 0; pp < PG / 2; ++pp) {
+        if (pp == FETCH_PAIR) fetch_step<P, PG, THREADS>(stage, a, pb0, min(step + 1, n_steps - 1), n_it, kvh, tid);
         const int it_a = step * PG + 2 * pp;
         if (it_a >= n_it) continue;
         const bool has_b = it_a + 1 < n_it;
