@@ -773,7 +773,7 @@ __device__ __forceinline__ void merge_wave_body(const MergeArgs &a, int kvh, int
     for (int i = 0; i < PER; ++i) {
         const bool ok = g + 16 * i < a.splits_total;
         const uint32_t oo = ok ? o0 + (uint32_t)(16 * i) * o_stride : o0;
-        ov[i] = *reinterpret_cast<const f32x4_t *>(po + oo);
+        ov[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(po + oo)); // read once
     }
     float mv[PER], lv[PER];
     float mx = -INFINITY;
